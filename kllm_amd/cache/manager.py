@@ -15,7 +15,8 @@ reservation here is all or nothing across every group.
 
 Pages are given back when a request is released, and, in a windowed group,
 as soon as every position of a page lies behind the window of every token
-still to come.  Pages are not cleared when they are handed out again; readers
+still to come; the pages of a group's kept first positions (``keep_first``)
+stay with the request.  Pages are not cleared when they are handed out again; readers
 never look beyond a request's own length.
 """
 
@@ -36,17 +37,19 @@ class GroupSpec:
     page_size: int
     num_pages: int
     window: int = 0  # 0: all keys are kept
+    keep_first: int = 0  # with a window: the first positions that stay readable behind it
 
 
-def window_pages(n_tokens: int, step_tokens: int, page_size: int, window: int) -> int:
+def window_pages(n_tokens: int, step_tokens: int, page_size: int, window: int, keep_first: int = 0) -> int:
     """Most pages a request of up to n_tokens holds in a group: all of its
     pages without a window; with one, the pages from the first key that the
     oldest token still to come may read to the end of the step being reserved:
-    at most ceil((step + window - 1) / page_size) + 1."""
+    at most ceil((step + window - 1) / page_size) + 1, and the pages of the kept
+    first positions."""
     whole = -(-n_tokens // page_size)
     if window <= 0:
         return whole
-    return min(whole, -(-(step_tokens + window - 1) // page_size) + 1)
+    return min(whole, -(-(step_tokens + window - 1) // page_size) + 1 + -(-keep_first // page_size))
 
 
 @dataclass
@@ -115,7 +118,7 @@ class CacheManager:
         (default: all of them at once).  A windowed group never holds more
         than its window and one step's tokens span."""
         step = n_tokens if step_tokens is None else max(1, min(int(step_tokens), n_tokens))
-        return [window_pages(n_tokens, step, grp.page_size, grp.window) for grp in self.groups]
+        return [window_pages(n_tokens, step, grp.page_size, grp.window, grp.keep_first) for grp in self.groups]
 
     # ------------------------------------------------------------ protocol
     def reserve(self, request_id: Hashable, n_tokens: int) -> None:
@@ -154,10 +157,12 @@ class CacheManager:
         rc.reserved -= n_tokens
         for g in range(len(self.groups)):
             first = min(self._first_needed_page(g, rc.length), len(rc.tables[g]))
-            if first > rc.first_live[g]:
-                gone = rc.tables[g][rc.first_live[g]:first]
+            kept = -(-self.groups[g].keep_first // self.groups[g].page_size)     # pages of the kept first positions
+            lo = max(rc.first_live[g], kept)
+            if first > lo:
+                gone = rc.tables[g][lo:first]
                 self.pools[g].free(gone)
-                for j in range(rc.first_live[g], first):
+                for j in range(lo, first):
                     rc.tables[g][j] = FREED
                 rc.first_live[g] = first
 
@@ -178,7 +183,7 @@ class CacheManager:
             "live_requests": len(self.requests),
             "free_slots": self.slots.free_slots,
             "groups": [
-                {"name": g.name, "page_size": g.page_size, "window": g.window,
+                {"name": g.name, "page_size": g.page_size, "window": g.window, "keep_first": g.keep_first,
                  "pages": p.num_pages, "used": p.used_pages, "free": p.free_pages,
                  "high_water": p.high_water}
                 for g, p in zip(self.groups, self.pools)],

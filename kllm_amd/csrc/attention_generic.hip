@@ -13,7 +13,8 @@
 // (vd); a chunked mask (chunk > 0: the query at p reads no key before
 // p - p % chunk, chunks counted from position 0 of the request); a sink
 // (sink != 0: the softmax's denominator has one more term, exp(0), a key whose
-// score is 0 and whose value is nothing).
+// score is 0 and whose value is nothing); kept first positions (keep_first > 0: the first
+// keep_first positions of a request stay readable behind the window, at their true places).
 //
 // Page layout: keys [KV][slot][hd], then values [KV][vd][slot].
 #include <math.h>
@@ -31,7 +32,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_generic_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ span_of_token,
     const int* __restrict__ block_table, int max_pages, int page_size, int H, int KV, int hd,
-    int vd, int window, int chunk, int sink, float scale, const float* __restrict__ slopes) {
+    int vd, int window, int chunk, int sink, float scale, const float* __restrict__ slopes, int keep_first) {
   __shared__ float qs[kMaxHeadDim];
   __shared__ float ps[kAttnThreads];
   __shared__ float red[16];
@@ -60,12 +61,17 @@ __global__ __launch_bounds__(kAttnThreads) void attn_generic_kernel(
   const int chunk_keys = chunk_pages * page_size;  // <= 256 (page_size <= 256 is checked on the host)
 
   float m = -INFINITY, l = 0.f, acc = 0.f;
-  for (int pg0 = start / page_size; pg0 * page_size < len; pg0 += chunk_pages) {
+  // Two runs of keys: the kept first positions that lie behind the window (none without
+  // keep_first), then the window itself.  Pages between the two may have been given back.
+  const int kept = min(keep_first, start);
+  for (int run = kept > 0 ? 0 : 1; run < 2; ++run) {
+  const int lo_key = run == 0 ? 0 : start, hi_key = run == 0 ? kept : len;
+  for (int pg0 = lo_key / page_size; pg0 * page_size < hi_key; pg0 += chunk_pages) {
     const int base = pg0 * page_size;
     // ---- scores of this chunk: thread i <-> key base + i
     float s = -INFINITY;
     const int key = base + tid;
-    if (tid < chunk_keys && key >= start && key < len) {
+    if (tid < chunk_keys && key >= lo_key && key < hi_key) {
       const int page = table[key / page_size];
       const T* krow = cache + page * page_elems + kvh * kblock + (long)(key % page_size) * hd;
       float dot = 0.f;
@@ -85,7 +91,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_generic_kernel(
     if (pv_thread) {
       for (int pg = sl; pg < chunk_pages; pg += nslice) {
         const int pbase = base + pg * page_size;
-        const int lo = max(start - pbase, 0), hi = min(len - pbase, page_size);
+        const int lo = max(lo_key - pbase, 0), hi = min(hi_key - pbase, page_size);
         if (lo >= hi) continue;
         const int page = table[pbase / page_size];
         const T* vrow = cache + page * page_elems + KV * kblock + kvh * vblock + (long)d * page_size;
@@ -94,6 +100,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_generic_kernel(
       }
     }
     __syncthreads();  // ps is rewritten by the next chunk
+  }
   }
 
   if (sink) {   // one more key whose score is 0: it joins the sum, and nothing else
@@ -119,7 +126,7 @@ extern "C" int kllm_attn_generic(const void* q, void* out, const void* cache, co
                                  const int* span_of_token, const int* block_table, int max_pages,
                                  int page_size, int n, int H, int KV, int hd, int vd, int window,
                                  int chunk, int sink, float scale, const float* slopes, int dtype,
-                                 hipStream_t stream) {
+                                 int keep_first, hipStream_t stream) {
   KLLM_REQUIRE(q && out && cache && positions && span_of_token && block_table,
                "attn_generic: null pointer");
   KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && H % KV == 0, "attn_generic: bad heads n=%d H=%d KV=%d", n,
@@ -129,18 +136,18 @@ extern "C" int kllm_attn_generic(const void* q, void* out, const void* cache, co
   KLLM_REQUIRE(page_size > 0 && page_size <= kAttnThreads && max_pages > 0,
                "attn_generic: page_size %d is outside [1, %d]", page_size, kAttnThreads);
   KLLM_REQUIRE(vd > 0 && vd <= kMaxHeadDim, "attn_generic: value width %d is outside [1, %d]", vd, kMaxHeadDim);
-  KLLM_REQUIRE(window >= 0 && chunk >= 0, "attn_generic: negative window or chunk");
+  KLLM_REQUIRE(window >= 0 && chunk >= 0 && keep_first >= 0, "attn_generic: negative window, chunk or keep_first");
   KLLM_REQUIRE(H <= 65535, "attn_generic: too many heads for the grid");
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "attn_generic: unknown dtype %d", dtype);
   const dim3 grid(n, H);
   if (dtype == DT_F32)
     hipLaunchKernelGGL(attn_generic_kernel<float>, grid, dim3(kAttnThreads), 0, stream,
                        (const float*)q, (float*)out, (const float*)cache, positions, span_of_token,
-                       block_table, max_pages, page_size, H, KV, hd, vd, window, chunk, sink, scale, slopes);
+                       block_table, max_pages, page_size, H, KV, hd, vd, window, chunk, sink, scale, slopes, keep_first);
   else
     hipLaunchKernelGGL(attn_generic_kernel<bf16_t>, grid, dim3(kAttnThreads), 0, stream,
                        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, positions,
-                       span_of_token, block_table, max_pages, page_size, H, KV, hd, vd, window, chunk, sink, scale, slopes);
+                       span_of_token, block_table, max_pages, page_size, H, KV, hd, vd, window, chunk, sink, scale, slopes, keep_first);
   KLLM_CHECK_LAUNCH("attn_generic");
   return 0;
 }

@@ -44,7 +44,8 @@ __device__ __forceinline__ float gate_act(float g, int act) {
 
 // Activations without a gate (kllm_unary_act): the gates' two, and xIELU, whose two constants
 // are learned: for z > 0, a_pos z^2 + z/2; otherwise (1/2 + a_neg) (exp(z) - 1 - z) + z/2.
-enum : int { ACT_XIELU = 2, ACT_TANH = 3, UNARY_ACT_COUNT = 4 };
+// The square of the rectifier: max(z, 0)^2.
+enum : int { ACT_XIELU = 2, ACT_TANH = 3, ACT_RELU_SQ = 4, UNARY_ACT_COUNT = 5 };
 
 __device__ __forceinline__ float softplus_f32(float v) { return v > 20.f ? v : log1pf(expf(v)); }
 
@@ -52,6 +53,10 @@ __device__ __forceinline__ float unary_act(float z, int act, float a_pos, float 
   if (act == ACT_XIELU)
     return z > 0.f ? fmaf(a_pos * z, z, 0.5f * z) : fmaf(0.5f + a_neg, expm1f(z) - z, 0.5f * z);
   if (act == ACT_TANH) return tanhf(z);
+  if (act == ACT_RELU_SQ) {
+    const float p = fmaxf(z, 0.f);
+    return p * p;
+  }
   return gate_act(z, act);
 }
 

@@ -18,14 +18,21 @@ constexpr int kThreads = 256;
 template <typename T>
 __global__ void embed_kernel(float* __restrict__ out, const T* __restrict__ table,
                              const int* __restrict__ ids, const int* __restrict__ from,
-                             const int* __restrict__ sampled, int d, int vocab) {
+                             const int* __restrict__ sampled, int d, int vocab, float scale,
+                             T* __restrict__ copy) {
   const long t = blockIdx.x;
   int id = ids[t];
   if (from && from[t] >= 0) id = sampled[from[t]];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // the host has checked the range
   const T* src = table + (long)id * d;
   float* dst = out + t * d;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) dst[i] = to_f32(src[i]);
+  // (a design may multiply the embedded row by a constant; the rows in the table's own type are
+  // left beside the 32-bit ones for a first sub-layer that reads the stream itself)
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    const float v = to_f32(src[i]) * scale;
+    dst[i] = v;
+    if (copy) copy[t * d + i] = from_f32<T>(v);
+  }
 }
 
 // Sum of the nsplit partial values p[0], p[stride], ...: eight loads are in
@@ -368,17 +375,18 @@ extern "C" int kllm_sum_splits(const float* in, int nsplit, long count, void* ou
 }
 
 extern "C" int kllm_embed(float* out, const void* table, const int* ids, const int* from,
-                          const int* sampled, int n, int d, int vocab, int dtype, hipStream_t stream) {
+                          const int* sampled, int n, int d, int vocab, int dtype, float scale, void* copy,
+                          hipStream_t stream) {
   KLLM_REQUIRE(out && table && ids, "embed: null pointer");
   KLLM_REQUIRE((from == nullptr) == (sampled == nullptr), "embed: from and sampled go together");
   KLLM_REQUIRE(n > 0 && d > 0 && vocab > 0, "embed: bad sizes n=%d d=%d vocab=%d", n, d, vocab);
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "embed: unknown dtype %d", dtype);
   if (dtype == DT_F32)
     hipLaunchKernelGGL(embed_kernel<float>, dim3(n), dim3(kThreads), 0, stream, out,
-                       (const float*)table, ids, from, sampled, d, vocab);
+                       (const float*)table, ids, from, sampled, d, vocab, scale, (float*)copy);
   else
     hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(n), dim3(kThreads), 0, stream, out,
-                       (const bf16_t*)table, ids, from, sampled, d, vocab);
+                       (const bf16_t*)table, ids, from, sampled, d, vocab, scale, (bf16_t*)copy);
   KLLM_CHECK_LAUNCH("embed");
   return 0;
 }

@@ -49,6 +49,17 @@ static const Op kOps[] = {
     KLLM_CMD_OP(kllm_moe_expert),
     KLLM_CMD_OP(kllm_moe_expert_rows),
     KLLM_CMD_OP(kllm_moe_combine),
+    KLLM_CMD_OP(kllm_conv_state_update),
+    KLLM_CMD_OP(kllm_gated_delta_prep),
+    KLLM_CMD_OP(kllm_gated_delta_scan),
+    KLLM_CMD_OP(kllm_linear_recurrence_prep),
+    KLLM_CMD_OP(kllm_linear_recurrence_scan),
+    KLLM_CMD_OP(kllm_latent_kv_append),
+    KLLM_CMD_OP(kllm_latent_norm),
+    KLLM_CMD_OP(kllm_latent_query),
+    KLLM_CMD_OP(kllm_attn_latent),
+    KLLM_CMD_OP(kllm_latent_out),
+    KLLM_CMD_OP(kllm_scaled_sum),
 };
 constexpr int kNumOps = (int)(sizeof(kOps) / sizeof(kOps[0]));
 

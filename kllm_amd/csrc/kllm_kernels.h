@@ -50,10 +50,11 @@ int kllm_calibrate_read(const void* src, long bytes, float* sink, hipStream_t st
 int kllm_calibrate_read_workgroups(void);
 int kllm_calibrate_mfma(int dtype, int iters, float* sink, double* flops, hipStream_t stream);
 
-/* out[t] = table[ids[t]]; with `from` (and `sampled`), token t whose from[t] >= 0 takes its id
- * from sampled[from[t]], a token id that an earlier launch left on the device. */
+/* out[t] = scale * table[ids[t]]; with `from` (and `sampled`), token t whose from[t] >= 0 takes its id
+ * from sampled[from[t]], a token id that an earlier launch left on the device.  `copy` (or null):
+ * the same rows in the table's own type. */
 int kllm_embed(float* out, const void* table, const int* ids, const int* from, const int* sampled,
-               int n, int d, int vocab, int dtype, hipStream_t stream);
+               int n, int d, int vocab, int dtype, float scale, void* copy, hipStream_t stream);
 
 /* v = x[src] + sum of the nsplit partial deltas (delta may be null);
  * x[src] = v when write_x; out[r] = rmsnorm(v) * w when out is not null.
@@ -212,11 +213,12 @@ int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOut* out, con
  * that grows with the distance to the key.
  * `vd`: width of a value (a page holds keys [KV][slot][hd], then values [KV][vd][slot]);
  * `chunk` > 0: the query at position p reads no key before p - p % chunk; `sink` != 0: the
- * softmax's denominator has one more term, exp(0). */
+ * softmax's denominator has one more term, exp(0); `keep_first` > 0: the first keep_first
+ * positions of a request stay readable behind the window (their pages are kept). */
 int kllm_attn_generic(const void* q, void* out, const void* cache, const int* positions,
                       const int* span_of_token, const int* block_table, int max_pages,
                       int page_size, int n, int H, int KV, int hd, int vd, int window, int chunk,
-                      int sink, float scale, const float* slopes, int dtype, hipStream_t stream);
+                      int sink, float scale, const float* slopes, int dtype, int keep_first, hipStream_t stream);
 
 /* Decode attention on the matrix cores: every token's keys are cut into
  * `nslices` slices (1..256) that run side by side (bfloat16: a workgroup of 4
@@ -286,6 +288,7 @@ int kllm_add_sinusoid(float* x, const int* positions, int n, int d, double base,
  * (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2. */
 #define KLLM_ACT_XIELU 2
 #define KLLM_ACT_TANH 3
+#define KLLM_ACT_RELU_SQ 4      /* max(z, 0)^2 */
 /* out[n][f] = act(sum over s of in[s][n][f]), rounded to out_dtype; a row of `in` begins every
  * in_row_stride elements (f if the rows follow each other). */
 int kllm_unary_act(const float* in, int nsplit, long split_stride, int in_row_stride, void* out, int out_dtype,
@@ -353,12 +356,16 @@ int kllm_rope_tables_freq(float* cos_t, float* sin_t, const int* positions, cons
  * `bias` (or null), turns the first `rot` elements of every query and key head (pairs (2j, 2j+1)
  * if `interleaved`, else (j, j + rot/2); cos/sin [n][rot/2] or null), divides every query and
  * key head by its root mean square (`unit_norm`, eps inside the root), writes the queries and
- * appends keys and values to the pages (keys [KV][slot][dk], then values [KV][dv][slot]). */
+ * appends keys and values to the pages (keys [KV][slot][dk], then values [KV][dv][slot]).
+ * With `q_weight` and `k_weight` ([dk] each, shared by the heads) the norm comes first and has
+ * weights: every query and key head is divided by its root mean square and multiplied by the
+ * weight, then rotated (`unit_norm` is then not looked at). */
 int kllm_qkv_norm_append(const float* qkv, int nsplit, long split_stride, const float* bias,
                          const float* cos_t, const float* sin_t, int rot, int interleaved, int unit_norm,
                          float eps, void* q_out, void* cache, const int* positions,
                          const int* span_of_token, const int* block_table, int max_pages, int page_size,
-                         int n, int H, int KV, int dk, int dv, int dtype, hipStream_t stream);
+                         int n, int H, int KV, int dk, int dv, int dtype, const float* q_weight,
+                         const float* k_weight, hipStream_t stream);
 /* out [n][f] = gated(g, u) of the float32 sums gu [nsplit][n][2 f] (gates, then ups) plus `bias`
  * [2 f] or null.  act: a gate's activation (act(g) u), or 4: with g' = min(g, limit) and u' =
  * clamp(u, -limit, limit), g' sigmoid(alpha g') (u' + 1). */
@@ -408,6 +415,65 @@ int kllm_sample(int* out, const float* logits, const float* temperature, const f
 int kllm_command_op(const char* name);
 int kllm_command_nargs(int op);
 int kllm_run_commands(const uint64_t* words, long n_words, int* failed, hipStream_t stream);
+
+/* ---- recurrent mixers with a short convolution (recurrent.hip) ----
+ * `proj` are float32 sums [nsplit][n][cols] of a step's projections.  A request's state is a run of
+ * `slot_stride` floats per slot; the pointers given here point at the field in slot 0. */
+
+/* The convolution's part of the state, [C][taps - 1] per slot: the inputs (columns col0 .. col0 + C of
+ * proj, plus in_bias [C] or null) of each span's last taps - 1 positions. */
+int kllm_conv_state_update(const float* proj, int nsplit, long split_stride, int cols, int col0, int C,
+                           const float* in_bias, float* state, long slot_stride, int taps, const int* slots,
+                           const int* span_start, const int* span_pos, int n_spans, hipStream_t stream);
+/* Gated delta rule, what the recurrence reads.  proj columns: q (G dk) | k (G dk) | v (H dv) | b (H) |
+ * a (H) | gate (H dv).  conv_w [2 G dk + H dv][taps]; state: the convolution's field.  Writes qn, kn
+ * [n][G dk] (unit vectors per head, qn times dk^-1/2), vv [n][H dv], gb [n][2][H] (decay, beta) and
+ * gate [n][H dv] = silu of the gate's sums. */
+int kllm_gated_delta_prep(const float* proj, int nsplit, long split_stride, const float* conv_w, int taps,
+                          const float* state, long slot_stride, const float* a_log, const float* dt_bias,
+                          const int* span_of_token, const int* slots, const int* span_start, const int* span_pos,
+                          float* qn, float* kn, float* vv, float* gb, float* gate, int n, int H, int G, int dk,
+                          int dv, float unit_eps, hipStream_t stream);
+int kllm_gated_delta_max_dim(void);
+/* The recurrence: state [H][dk][dv] per slot, o_out [n][H dv]. */
+int kllm_gated_delta_scan(const float* qn, const float* kn, const float* vv, const float* gb, float* o_out,
+                          float* state, long slot_stride, const int* slots, const int* span_start,
+                          const int* span_pos, int n_spans, int H, int G, int dk, int dv, hipStream_t stream);
+/* Gated linear recurrence.  proj columns: y (W) | x (W).  wr_t, wi_t: the gates' block-diagonal matrices
+ * [blocks][in][out]; rate [W] = 8 softplus(lambda).  Writes a and the added term, [n][W] each. */
+int kllm_linear_recurrence_prep(const float* proj, int nsplit, long split_stride, const float* x_bias,
+                                const float* conv_w, const float* conv_b, int taps, const float* state,
+                                long slot_stride, const float* wr_t, const float* wi_t, const float* br,
+                                const float* bi, const float* rate, const int* span_of_token, const int* slots,
+                                const int* span_start, const int* span_pos, float* a_out, float* b_out, int n, int W,
+                                int blocks, hipStream_t stream);
+/* S <- a S + b per span and channel (state [W] per slot); out [n][W] = S * gelu_tanh(y + y_bias). */
+int kllm_linear_recurrence_scan(const float* a_in, const float* b_in, const float* proj, int nsplit,
+                                long split_stride, const float* y_bias, float* state, long slot_stride,
+                                const int* slots, const int* span_start, const int* span_pos, void* out, int n_spans,
+                                int W, int dtype, hipStream_t stream);
+
+/* out[i] = sa * sum over a's slices + sb * sum over b's slices (float32, `count` elements a slice). */
+int kllm_scaled_sum(float* out, const float* a, int na, long stride_a, float sa, const float* b, int nb,
+                    long stride_b, float sb, long count, hipStream_t stream);
+
+/* ---- attention through low-rank latents (latent.hip): one cached row of rank + dr per token ---- */
+int kllm_latent_max_row(void);
+int kllm_latent_kv_append(const float* dkv, int nsplit, long split_stride, const float* weight, float eps,
+                          const float* cos_t, const float* sin_t, void* cache, const int* positions,
+                          const int* span_of_token, const int* block_table, int max_pages, int page_size, int n,
+                          int rank, int dr, int dtype, long in_stride, hipStream_t stream);
+/* out [n][r] = RMS norm with `weight` of r columns of float32 sums whose rows are in_stride apart. */
+int kllm_latent_norm(const float* in, int nsplit, long split_stride, long in_stride, const float* weight, float eps,
+                     void* out, int n, int r, int dtype, hipStream_t stream);
+int kllm_latent_query(const float* q, int nsplit, long split_stride, const void* w_uk, const float* cos_t,
+                      const float* sin_t, void* out, int n, int H, int d, int dr, int rank, int dtype,
+                      hipStream_t stream);
+int kllm_attn_latent(const void* q, void* out, const void* cache, const int* positions, const int* span_of_token,
+                     const int* block_table, int max_pages, int page_size, int n, int H, int row, int rank,
+                     float scale, int dtype, hipStream_t stream);
+int kllm_latent_out(const void* attended, const void* w_uv, const float* gate, int nsplit, long split_stride,
+                    long gate_stride, void* out, int n, int H, int dv, int rank, int dtype, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,310 @@
+// Attention through low-rank latents.  Per token one vector is cached for all heads: the
+// normalised latent c [rank] followed by one rotated key part [dr].  A head's key is
+// [W_uk,h c | rotated part] and its value W_uv,h c, so with the query's unrotated part folded
+// through W_uk,h (q' = W_uk,h^T q, [rank]) the score is q' . c + q_rot . k_rot, the weighted
+// sum over the keys is taken of c itself, and W_uv,h is applied once to that sum:
+//
+//   latent_kv_append   sums of W_dkv h -> RMS norm (weights) of the first rank, rotation of the
+//                      last dr (halves paired), appended to the pages (one row of rank + dr a slot)
+//   latent_query       sums of W_uq c_q -> per head [W_uk,h^T q_h | rotated q_h], rank + dr wide
+//   attn_latent        one workgroup a (token, head): online softmax over 256 keys at a time,
+//                      the values being the first rank elements of the cached rows
+//   latent_out         per head W_uv,h times the attended latent, times sigmoid of the gate's sums
+//
+// Scores, softmax, norms and rotation are 32-bit; the cached rows, the folded queries and the
+// attended latents are stored in the compute type.
+#include <math.h>
+
+#include "common.hpp"
+#include "kllm_kernels.h"
+
+namespace kllm {
+
+constexpr int kLatThreads = 256;
+constexpr int kLatMaxRow = 1024;       // rank + dr of a cached row
+constexpr int kLatMaxPer = kLatMaxRow / kLatThreads;
+
+template <typename T>
+__global__ __launch_bounds__(kLatThreads) void latent_kv_append_kernel(
+    const float* __restrict__ dkv, int nsplit, long split_stride, const float* __restrict__ weight, float eps,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, T* __restrict__ cache,
+    const int* __restrict__ positions, const int* __restrict__ span_of_token, const int* __restrict__ block_table,
+    int max_pages, int page_size, int rank, int dr, long in_stride) {
+  __shared__ float red[16];
+  const long t = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int row = rank + dr, half = dr / 2;
+  const float* in = dkv + t * in_stride;
+  const int pos = positions[t];
+  const long page = block_table[(long)span_of_token[t] * max_pages + pos / page_size];
+  T* dst = cache + (page * page_size + pos % page_size) * row;
+  float v[kLatMaxPer];
+  float ss = 0.f;
+#pragma unroll
+  for (int q = 0; q < kLatMaxPer; ++q) {
+    const int i = tid + q * kLatThreads;
+    v[q] = 0.f;
+    if (i < rank) {
+      for (int s = 0; s < nsplit; ++s) v[q] += in[s * split_stride + i];
+      ss = fmaf(v[q], v[q], ss);
+    }
+  }
+  const float rstd = 1.f / sqrtf(block_sum(ss, red) / (float)rank + eps);
+#pragma unroll
+  for (int q = 0; q < kLatMaxPer; ++q) {
+    const int i = tid + q * kLatThreads;
+    if (i < rank) dst[i] = from_f32<T>(v[q] * rstd * weight[i]);
+  }
+  for (int i = tid; i < half; i += kLatThreads) {
+    float a = 0.f, b = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      a += in[s * split_stride + rank + i];
+      b += in[s * split_stride + rank + half + i];
+    }
+    const float c = cos_t[t * half + i], sn = sin_t[t * half + i];
+    dst[rank + i] = from_f32<T>(a * c - b * sn);
+    dst[rank + half + i] = from_f32<T>(b * c + a * sn);
+  }
+}
+
+// out [n][r] = N(in row's r elements) * weight, the rows of `in` in_stride apart; one workgroup a row.
+template <typename T>
+__global__ __launch_bounds__(kLatThreads) void latent_norm_kernel(const float* __restrict__ in, int nsplit,
+                                                                  long split_stride, long in_stride,
+                                                                  const float* __restrict__ weight, float eps,
+                                                                  T* __restrict__ out, int r) {
+  __shared__ float red[16];
+  const long t = blockIdx.x;
+  const int tid = threadIdx.x;
+  const float* src = in + t * in_stride;
+  float ss = 0.f;
+  for (int i = tid; i < r; i += kLatThreads) {
+    float v = 0.f;
+    for (int s = 0; s < nsplit; ++s) v += src[s * split_stride + i];
+    ss = fmaf(v, v, ss);
+  }
+  const float rstd = 1.f / sqrtf(block_sum(ss, red) / (float)r + eps);
+  for (int i = tid; i < r; i += kLatThreads) {
+    float v = 0.f;
+    for (int s = 0; s < nsplit; ++s) v += src[s * split_stride + i];
+    out[t * r + i] = from_f32<T>(v * rstd * weight[i]);
+  }
+}
+
+// q: [nsplit][n][H * (d + dr)], a head laid out [d unrotated | dr rotated]; w_uk [H * d][rank].
+template <typename T>
+__global__ __launch_bounds__(kLatThreads) void latent_query_kernel(
+    const float* __restrict__ q, int nsplit, long split_stride, const T* __restrict__ w_uk,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, T* __restrict__ out, int H, int d, int dr,
+    int rank) {
+  extern __shared__ float qh[];          // [d + dr]
+  const long t = blockIdx.x;
+  const int h = blockIdx.y, tid = threadIdx.x;
+  const int hw = d + dr, half = dr / 2;
+  const float* in = q + (t * H + h) * hw;
+  for (int i = tid; i < hw; i += kLatThreads) {
+    float v = 0.f;
+    for (int s = 0; s < nsplit; ++s) v += in[s * split_stride + i];
+    qh[i] = v;
+  }
+  __syncthreads();
+  T* dst = out + (t * H + h) * (rank + dr);
+  const T* w = w_uk + (long)h * d * rank;
+  for (int r = tid; r < rank; r += kLatThreads) {
+    float acc = 0.f;
+    for (int i = 0; i < d; ++i) acc = fmaf(qh[i], to_f32(w[(long)i * rank + r]), acc);
+    dst[r] = from_f32<T>(acc);
+  }
+  for (int i = tid; i < half; i += kLatThreads) {
+    const float a = qh[d + i], b = qh[d + half + i];
+    const float c = cos_t[t * half + i], sn = sin_t[t * half + i];
+    dst[rank + i] = from_f32<T>(a * c - b * sn);
+    dst[rank + half + i] = from_f32<T>(b * c + a * sn);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kLatThreads) void attn_latent_kernel(
+    const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ cache, const int* __restrict__ positions,
+    const int* __restrict__ span_of_token, const int* __restrict__ block_table, int max_pages, int page_size, int H,
+    int row, int rank, float scale) {
+  __shared__ float qs[kLatMaxRow];
+  __shared__ float ps[kLatThreads];
+  __shared__ float red[16];
+  const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int len = positions[t] + 1;
+  const int* table = block_table + (long)span_of_token[t] * max_pages;
+  const T* qrow = q + ((long)t * H + h) * row;
+  for (int i = tid; i < row; i += kLatThreads) qs[i] = to_f32(qrow[i]);
+  __syncthreads();
+  float m = -INFINITY, l = 0.f;
+  float acc[kLatMaxPer];
+#pragma unroll
+  for (int c = 0; c < kLatMaxPer; ++c) acc[c] = 0.f;
+  for (int base = 0; base < len; base += kLatThreads) {
+    const int key = base + tid;
+    float s = -INFINITY;
+    if (key < len) {
+      const T* krow = cache + ((long)table[key / page_size] * page_size + key % page_size) * row;
+      float dot = 0.f;
+      for (int i = 0; i < row; ++i) dot = fmaf(qs[i], to_f32(krow[i]), dot);
+      s = dot * scale;
+    }
+    const float m_new = fmaxf(m, block_max(s, red));
+    const float alpha = expf(m - m_new);
+    const float p = (s == -INFINITY) ? 0.f : expf(s - m_new);
+    ps[tid] = p;
+    l = l * alpha + block_sum(p, red);       // its barriers also publish ps
+    m = m_new;
+    const int nk = min(kLatThreads, len - base);
+#pragma unroll
+    for (int c = 0; c < kLatMaxPer; ++c) {
+      const int e = tid + c * kLatThreads;
+      acc[c] *= alpha;
+      if (e < rank) {
+        float a = acc[c];
+        int pg = -1;
+        const T* prow = nullptr;
+        for (int k = 0; k < nk; ++k) {
+          const int kk = base + k;
+          if (kk / page_size != pg) {
+            pg = kk / page_size;
+            prow = cache + (long)table[pg] * page_size * row;
+          }
+          a = fmaf(ps[k], to_f32(prow[(long)(kk % page_size) * row + e]), a);
+        }
+        acc[c] = a;
+      }
+    }
+    __syncthreads();                         // ps is rewritten by the next round
+  }
+#pragma unroll
+  for (int c = 0; c < kLatMaxPer; ++c) {
+    const int e = tid + c * kLatThreads;
+    if (e < rank) out[((long)t * H + h) * rank + e] = from_f32<T>(acc[c] / l);
+  }
+}
+
+// attended: [n][H][rank]; w_uv [H * dv][rank]; gate: [nsplit][n][H * dv] sums or null.
+template <typename T>
+__global__ __launch_bounds__(kLatThreads) void latent_out_kernel(
+    const T* __restrict__ attended, const T* __restrict__ w_uv, const float* __restrict__ gate, int nsplit,
+    long split_stride, long gate_stride, T* __restrict__ out, int H, int dv, int rank) {
+  extern __shared__ float al[];          // [rank]
+  const long t = blockIdx.x;
+  const int h = blockIdx.y, tid = threadIdx.x;
+  const T* src = attended + (t * H + h) * rank;
+  for (int i = tid; i < rank; i += kLatThreads) al[i] = to_f32(src[i]);
+  __syncthreads();
+  for (int j = tid; j < dv; j += kLatThreads) {
+    const T* w = w_uv + ((long)h * dv + j) * rank;
+    float acc = 0.f;
+    for (int r = 0; r < rank; ++r) acc = fmaf(al[r], to_f32(w[r]), acc);
+    const long col = (long)h * dv + j;
+    if (gate) {
+      float g = 0.f;
+      for (int s = 0; s < nsplit; ++s) g += gate[s * split_stride + t * gate_stride + col];
+      acc *= sigmoid_f32(g);
+    }
+    out[t * H * dv + col] = from_f32<T>(acc);
+  }
+}
+
+}  // namespace kllm
+
+using namespace kllm;
+
+extern "C" int kllm_latent_max_row(void) { return kLatMaxRow; }
+
+extern "C" int kllm_latent_kv_append(const float* dkv, int nsplit, long split_stride, const float* weight, float eps,
+                                     const float* cos_t, const float* sin_t, void* cache, const int* positions,
+                                     const int* span_of_token, const int* block_table, int max_pages, int page_size,
+                                     int n, int rank, int dr, int dtype, long in_stride, hipStream_t stream) {
+  KLLM_REQUIRE(dkv && weight && cos_t && sin_t && cache && positions && span_of_token && block_table,
+               "latent_kv_append: null pointer");
+  KLLM_REQUIRE(n > 0 && nsplit >= 1 && rank > 0 && dr > 0 && dr % 2 == 0 && rank + dr <= kLatMaxRow,
+               "latent_kv_append: bad sizes n=%d rank=%d dr=%d (rows of up to %d)", n, rank, dr, kLatMaxRow);
+  KLLM_REQUIRE(max_pages > 0 && page_size > 0, "latent_kv_append: bad cache sizes");
+  KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "latent_kv_append: unknown dtype %d", dtype);
+  if (dtype == DT_F32)
+    hipLaunchKernelGGL(latent_kv_append_kernel<float>, dim3(n), dim3(kLatThreads), 0, stream, dkv, nsplit, split_stride,
+                       weight, eps, cos_t, sin_t, (float*)cache, positions, span_of_token, block_table, max_pages,
+                       page_size, rank, dr, in_stride);
+  else
+    hipLaunchKernelGGL(latent_kv_append_kernel<bf16_t>, dim3(n), dim3(kLatThreads), 0, stream, dkv, nsplit,
+                       split_stride, weight, eps, cos_t, sin_t, (bf16_t*)cache, positions, span_of_token, block_table,
+                       max_pages, page_size, rank, dr, in_stride);
+  KLLM_CHECK_LAUNCH("latent_kv_append");
+  return 0;
+}
+
+extern "C" int kllm_latent_norm(const float* in, int nsplit, long split_stride, long in_stride, const float* weight,
+                                float eps, void* out, int n, int r, int dtype, hipStream_t stream) {
+  KLLM_REQUIRE(in && weight && out && n > 0 && r > 0 && nsplit >= 1 && in_stride >= r, "latent_norm: null pointer or bad sizes");
+  KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "latent_norm: unknown dtype %d", dtype);
+  if (dtype == DT_F32)
+    hipLaunchKernelGGL(latent_norm_kernel<float>, dim3(n), dim3(kLatThreads), 0, stream, in, nsplit, split_stride,
+                       in_stride, weight, eps, (float*)out, r);
+  else
+    hipLaunchKernelGGL(latent_norm_kernel<bf16_t>, dim3(n), dim3(kLatThreads), 0, stream, in, nsplit, split_stride,
+                       in_stride, weight, eps, (bf16_t*)out, r);
+  KLLM_CHECK_LAUNCH("latent_norm");
+  return 0;
+}
+
+extern "C" int kllm_latent_query(const float* q, int nsplit, long split_stride, const void* w_uk, const float* cos_t,
+                                 const float* sin_t, void* out, int n, int H, int d, int dr, int rank, int dtype,
+                                 hipStream_t stream) {
+  KLLM_REQUIRE(q && w_uk && cos_t && sin_t && out, "latent_query: null pointer");
+  KLLM_REQUIRE(n > 0 && nsplit >= 1 && H > 0 && H <= 65535 && d > 0 && dr > 0 && dr % 2 == 0 && rank > 0 &&
+                   rank + dr <= kLatMaxRow && d + dr <= 4096,
+               "latent_query: bad sizes n=%d H=%d d=%d dr=%d rank=%d", n, H, d, dr, rank);
+  KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "latent_query: unknown dtype %d", dtype);
+  const size_t lds = (size_t)(d + dr) * sizeof(float);
+  if (dtype == DT_F32)
+    hipLaunchKernelGGL(latent_query_kernel<float>, dim3(n, H), dim3(kLatThreads), lds, stream, q, nsplit, split_stride,
+                       (const float*)w_uk, cos_t, sin_t, (float*)out, H, d, dr, rank);
+  else
+    hipLaunchKernelGGL(latent_query_kernel<bf16_t>, dim3(n, H), dim3(kLatThreads), lds, stream, q, nsplit, split_stride,
+                       (const bf16_t*)w_uk, cos_t, sin_t, (bf16_t*)out, H, d, dr, rank);
+  KLLM_CHECK_LAUNCH("latent_query");
+  return 0;
+}
+
+extern "C" int kllm_attn_latent(const void* q, void* out, const void* cache, const int* positions,
+                                const int* span_of_token, const int* block_table, int max_pages, int page_size, int n,
+                                int H, int row, int rank, float scale, int dtype, hipStream_t stream) {
+  KLLM_REQUIRE(q && out && cache && positions && span_of_token && block_table, "attn_latent: null pointer");
+  KLLM_REQUIRE(n > 0 && H > 0 && H <= 65535 && rank > 0 && rank <= row && row <= kLatMaxRow,
+               "attn_latent: bad sizes n=%d H=%d row=%d rank=%d (rows of up to %d)", n, H, row, rank, kLatMaxRow);
+  KLLM_REQUIRE(max_pages > 0 && page_size > 0, "attn_latent: bad cache sizes");
+  KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "attn_latent: unknown dtype %d", dtype);
+  if (dtype == DT_F32)
+    hipLaunchKernelGGL(attn_latent_kernel<float>, dim3(n, H), dim3(kLatThreads), 0, stream, (const float*)q,
+                       (float*)out, (const float*)cache, positions, span_of_token, block_table, max_pages, page_size, H,
+                       row, rank, scale);
+  else
+    hipLaunchKernelGGL(attn_latent_kernel<bf16_t>, dim3(n, H), dim3(kLatThreads), 0, stream, (const bf16_t*)q,
+                       (bf16_t*)out, (const bf16_t*)cache, positions, span_of_token, block_table, max_pages, page_size,
+                       H, row, rank, scale);
+  KLLM_CHECK_LAUNCH("attn_latent");
+  return 0;
+}
+
+extern "C" int kllm_latent_out(const void* attended, const void* w_uv, const float* gate, int nsplit, long split_stride,
+                               long gate_stride, void* out, int n, int H, int dv, int rank, int dtype,
+                               hipStream_t stream) {
+  KLLM_REQUIRE(attended && w_uv && out, "latent_out: null pointer");
+  KLLM_REQUIRE(n > 0 && H > 0 && H <= 65535 && dv > 0 && rank > 0 && rank <= 8192 && (!gate || nsplit >= 1),
+               "latent_out: bad sizes n=%d H=%d dv=%d rank=%d", n, H, dv, rank);
+  KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "latent_out: unknown dtype %d", dtype);
+  const size_t lds = (size_t)rank * sizeof(float);
+  if (dtype == DT_F32)
+    hipLaunchKernelGGL(latent_out_kernel<float>, dim3(n, H), dim3(kLatThreads), lds, stream, (const float*)attended,
+                       (const float*)w_uv, gate, nsplit, split_stride, gate_stride, (float*)out, H, dv, rank);
+  else
+    hipLaunchKernelGGL(latent_out_kernel<bf16_t>, dim3(n, H), dim3(kLatThreads), lds, stream, (const bf16_t*)attended,
+                       (const bf16_t*)w_uv, gate, nsplit, split_stride, gate_stride, (bf16_t*)out, H, dv, rank);
+  KLLM_CHECK_LAUNCH("latent_out");
+  return 0;
+}

@@ -1,0 +1,443 @@
+// Recurrent mixers whose state is carried from token to token, and what they share.
+//
+// A short causal convolution per channel: y_t = sum_j w[c][j] x_(t - taps + 1 + j), zeros before
+// position 0.  Its inputs of the last taps - 1 positions are part of a request's state: the
+// kernels that convolve read them for the first tokens of a span, and `conv_state_update`, a
+// launch of its own behind them, writes the span's last inputs there (one thread per request
+// and channel reads the old entries before it writes the new ones).
+//
+// The gated delta rule, per head with a state S [key channel][value channel]:
+//
+//   S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
+//
+// with q and k unit vectors per head (q also times dk^-1/2), g = exp(-exp(A) softplus(a + dt))
+// and beta = sigmoid(b).  `gated_delta_prep` turns the projections' sums into these (per token,
+// parallel: convolution and SiLU of q, k, v, the unit norms, g, beta and the output gate),
+// `gated_delta_scan` runs the recurrence (per request, head and block of value channels, token
+// after token); the output's norm and gate are kllm_delta_out's.
+//
+// The gated linear recurrence, per channel: with u the convolved input, gates
+// r = sigmoid(A_r u + b_r), i = sigmoid(A_i u + b_i) through block-diagonal matrices,
+// log a = -c r (c = 8 softplus(lambda), prepared once), S <- a S + sqrt(1 - a^2) i u, and the
+// output S * gelu(y) with y a second branch.  `linear_recurrence_prep` makes a and the added term
+// for every token (parallel), `linear_recurrence_scan` runs the chain.
+//
+// States are 32-bit and start from zero where a span's first position is 0.  Everything here
+// computes in 32-bit from the projections' 32-bit sums.
+#include <math.h>
+
+#include "common.hpp"
+#include "kllm_kernels.h"
+
+namespace kllm {
+
+constexpr int kRecThreads = 256;
+constexpr int kMaxTaps = 16;
+
+// The input of the convolution at row `row` of the step (a token of the same span), channel c.
+__device__ __forceinline__ float conv_input(const float* __restrict__ proj, int nsplit, long split_stride, long cols,
+                                            long col, const float* __restrict__ bias, long row) {
+  const float* p = proj + row * cols + col;
+  float v = 0.f;
+  for (int s = 0; s < nsplit; ++s) v += p[s * split_stride];
+  return bias ? v + bias[col] : v;
+}
+
+// The convolution's output for the token at row t (span rows from t0, `fresh`: the span starts at
+// position 0), channel c of C, whose input column is col0 + c; `st` is the request's
+// [C][taps - 1] entries.
+__device__ __forceinline__ float conv_at(const float* __restrict__ proj, int nsplit, long split_stride, long cols,
+                                         long col, const float* __restrict__ in_bias,
+                                         const float* __restrict__ w_row, int taps, const float* __restrict__ st_row,
+                                         bool fresh, long t, long t0) {
+  float y = 0.f;
+  const int K = taps - 1;
+  for (int j = 0; j < taps; ++j) {
+    const long row = t - K + j;
+    float x;
+    if (row >= t0) x = conv_input(proj, nsplit, split_stride, cols, col, in_bias, row);
+    else x = fresh ? 0.f : st_row[K - (int)(t0 - row)];
+    y = fmaf(w_row[j], x, y);
+  }
+  return y;
+}
+
+__global__ __launch_bounds__(kRecThreads) void conv_state_update_kernel(
+    const float* __restrict__ proj, int nsplit, long split_stride, long cols, int col0, int C,
+    const float* __restrict__ in_bias, float* __restrict__ state, long slot_stride, int taps,
+    const int* __restrict__ slots, const int* __restrict__ span_start, const int* __restrict__ span_pos) {
+  const int c = blockIdx.x * kRecThreads + threadIdx.x;
+  if (c >= C) return;
+  const int span = blockIdx.y;
+  const int K = taps - 1;
+  const long t0 = span_start[span], t1 = span_start[span + 1];
+  const long len = t1 - t0;
+  const bool fresh = span_pos[span] == 0;
+  float* st = state + (long)slots[span] * slot_stride + (long)c * K;
+  float old[kMaxTaps];
+  for (int j = 0; j < K; ++j) old[j] = fresh ? 0.f : st[j];
+  for (int j = 0; j < K; ++j) {
+    const long row = t1 - K + j;
+    st[j] = row >= t0 ? conv_input(proj, nsplit, split_stride, cols, col0 + c, in_bias, row) : old[j + len];
+  }
+}
+
+// ---------------------------------------------------------------------------- gated delta rule
+
+// proj: [nsplit][n][cols], columns q (G*dk) | k (G*dk) | v (H*dv) | b (H) | a (H) | gate (H*dv).
+// One workgroup a token.  Dynamic LDS: the convolved q, k, v of the token, [2*G*dk + H*dv] floats.
+__global__ __launch_bounds__(kRecThreads) void gated_delta_prep_kernel(
+    const float* __restrict__ proj, int nsplit, long split_stride, const float* __restrict__ conv_w, int taps,
+    const float* __restrict__ state, long slot_stride, const float* __restrict__ a_log,
+    const float* __restrict__ dt_bias, const int* __restrict__ span_of_token, const int* __restrict__ slots,
+    const int* __restrict__ span_start, const int* __restrict__ span_pos, float* __restrict__ qn,
+    float* __restrict__ kn, float* __restrict__ vv, float* __restrict__ gb, float* __restrict__ gate, int H, int G,
+    int dk, int dv, float unit_eps) {
+  extern __shared__ float vals[];
+  const long t = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int QK = G * dk, HV = H * dv, C = 2 * QK + HV;
+  const long cols = (long)C + 2 * H + HV;
+  const int span = span_of_token[t];
+  const long t0 = span_start[span];
+  const bool fresh = span_pos[span] == 0;
+  const float* st = state + (long)slots[span] * slot_stride;
+  for (int c = tid; c < C; c += kRecThreads) {
+    const float y = conv_at(proj, nsplit, split_stride, cols, c, nullptr, conv_w + (long)c * taps, taps,
+                            st + (long)c * (taps - 1), fresh, t, t0);
+    vals[c] = y / (1.f + expf(-y));                       // SiLU
+  }
+  __syncthreads();
+  // a wave a head of q or k: the unit norm
+  for (int item = wave; item < 2 * G; item += kRecThreads / kWave) {
+    const float* src = vals + (long)item * dk;
+    float ss = 0.f;
+    for (int e = lane; e < dk; e += kWave) ss = fmaf(src[e], src[e], ss);
+    ss = wave_sum(ss);
+    const bool is_q = item < G;
+    const float f = (is_q ? 1.f / sqrtf((float)dk) : 1.f) / sqrtf(ss + unit_eps);
+    float* dst = (is_q ? qn + t * QK + (long)item * dk : kn + t * QK + (long)(item - G) * dk);
+    for (int e = lane; e < dk; e += kWave) dst[e] = src[e] * f;
+  }
+  for (int c = tid; c < HV; c += kRecThreads) {
+    vv[t * HV + c] = vals[2 * QK + c];
+    float g = 0.f;
+    for (int s = 0; s < nsplit; ++s) g += proj[s * split_stride + t * cols + C + 2 * H + c];
+    gate[t * HV + c] = g / (1.f + expf(-g));
+  }
+  for (int h = tid; h < H; h += kRecThreads) {
+    float b = 0.f, a = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      b += proj[s * split_stride + t * cols + C + h];
+      a += proj[s * split_stride + t * cols + C + H + h];
+    }
+    gb[t * 2 * H + h] = expf(-expf(a_log[h]) * softplus_f32(a + dt_bias[h]));
+    gb[t * 2 * H + H + h] = sigmoid_f32(b);
+  }
+}
+
+constexpr int kDeltaParts = 16;                              // lanes that share a column of the state
+constexpr int kDeltaCols = kRecThreads / kDeltaParts;        // columns of a workgroup
+constexpr int kDeltaBlock = 16;                              // tokens staged at a time
+
+// Thread (j, p): column j of the workgroup's block of value channels, rows p, p + 16, ... of it.
+// A block of tokens' vectors goes through LDS: k and q [TB][dk] each, v [TB][16 columns], g and
+// beta [TB]; the sums over a column's rows are lane exchanges within its sixteen lanes.
+template <int NR>
+__global__ __launch_bounds__(kRecThreads) void gated_delta_scan_kernel(
+    const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vv,
+    const float* __restrict__ gb, float* __restrict__ o_out, float* __restrict__ state, long slot_stride,
+    const int* __restrict__ slots, const int* __restrict__ span_start, const int* __restrict__ span_pos, int H, int G,
+    int dk, int dv) {
+  extern __shared__ float lds[];
+  float* ks = lds;                                   // [TB][dk]
+  float* qs = ks + kDeltaBlock * dk;                 // [TB][dk]
+  float* vs = qs + kDeltaBlock * dk;                 // [TB][kDeltaCols]
+  float* gs = vs + kDeltaBlock * kDeltaCols;         // [TB][2]
+  const int span = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int g = h / (H / G);
+  const int jl = tid / kDeltaParts, p = tid % kDeltaParts;
+  const int j = blockIdx.z * kDeltaCols + jl;
+  const bool col = j < dv;
+  const long t0 = span_start[span], t1 = span_start[span + 1];
+  const bool fresh = span_pos[span] == 0;
+  float* S = state + (long)slots[span] * slot_stride + (long)h * dk * dv;
+  float s[NR];
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    const int r = p + kDeltaParts * i;
+    s[i] = (col && r < dk && !fresh) ? S[(long)r * dv + j] : 0.f;
+  }
+  const int QK = G * dk, HV = H * dv;
+  for (long tb = t0; tb < t1; tb += kDeltaBlock) {
+    const int nt = (int)min((long)kDeltaBlock, t1 - tb);
+    __syncthreads();                                 // the block before this one has been read
+    for (int i = tid; i < nt * dk; i += kRecThreads) {
+      const int tt = i / dk, e = i % dk;
+      ks[i] = kn[(tb + tt) * QK + (long)g * dk + e];
+      qs[i] = qn[(tb + tt) * QK + (long)g * dk + e];
+    }
+    for (int i = tid; i < nt * kDeltaCols; i += kRecThreads) {
+      const int tt = i / kDeltaCols, c = blockIdx.z * kDeltaCols + i % kDeltaCols;
+      vs[i] = c < dv ? vv[(tb + tt) * HV + (long)h * dv + c] : 0.f;
+    }
+    for (int i = tid; i < nt * 2; i += kRecThreads) gs[i] = gb[(tb + i / 2) * 2 * H + (i % 2) * H + h];
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float decay = gs[2 * tt], beta = gs[2 * tt + 1];
+      const float* kt = ks + tt * dk;
+      const float* qt = qs + tt * dk;
+      float kr[NR], dot = 0.f;
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        const int r = p + kDeltaParts * i;
+        kr[i] = r < dk ? kt[r] : 0.f;
+        s[i] *= decay;
+        dot = fmaf(s[i], kr[i], dot);
+      }
+#pragma unroll
+      for (int off = 1; off < kDeltaParts; off <<= 1) dot += __shfl_xor(dot, off, kWave);
+      const float u = beta * (vs[tt * kDeltaCols + jl] - dot);
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        const int r = p + kDeltaParts * i;
+        s[i] = fmaf(kr[i], u, s[i]);
+        o = fmaf(s[i], r < dk ? qt[r] : 0.f, o);
+      }
+#pragma unroll
+      for (int off = 1; off < kDeltaParts; off <<= 1) o += __shfl_xor(o, off, kWave);
+      if (col && p == 0) o_out[(tb + tt) * HV + (long)h * dv + j] = o;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    const int r = p + kDeltaParts * i;
+    if (col && r < dk) S[(long)r * dv + j] = s[i];
+  }
+}
+
+// ---------------------------------------------------------------------------- gated linear recurrence
+
+constexpr int kGateTokens = 8;       // tokens of a tile of the gates' products
+
+// proj: [nsplit][n][2 W], columns y | x.  Workgroup (tile of tokens, block b of the gates): the
+// convolved inputs of the block's channels for the tile's tokens go into LDS [TT][bs]; a thread
+// takes output channel o of the block for all the tile's tokens, the gates' matrices are read
+// [block][in][out] so that neighbouring threads read neighbouring weights.
+__global__ __launch_bounds__(kRecThreads) void linear_recurrence_prep_kernel(
+    const float* __restrict__ proj, int nsplit, long split_stride, const float* __restrict__ x_bias,
+    const float* __restrict__ conv_w, const float* __restrict__ conv_b, int taps, const float* __restrict__ state,
+    long slot_stride, const float* __restrict__ wr_t, const float* __restrict__ wi_t, const float* __restrict__ br,
+    const float* __restrict__ bi, const float* __restrict__ rate, const int* __restrict__ span_of_token,
+    const int* __restrict__ slots, const int* __restrict__ span_start, const int* __restrict__ span_pos,
+    float* __restrict__ a_out, float* __restrict__ b_out, int n, int W, int bs) {
+  extern __shared__ float us[];                      // [TT][bs]
+  const int tile = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const long tfirst = (long)tile * kGateTokens;
+  const int nt = (int)min((long)kGateTokens, n - tfirst);
+  const long cols = 2L * W;
+  for (int i = tid; i < nt * bs; i += kRecThreads) {
+    const int tt = i / bs, c = b * bs + i % bs;
+    const long t = tfirst + tt;
+    const int span = span_of_token[t];
+    // (the convolution's input carries the projection's bias; before position 0 it is zero)
+    us[i] = conv_at(proj, nsplit, split_stride, cols, W + c, x_bias - W, conv_w + (long)c * taps, taps,
+                    state + (long)slots[span] * slot_stride + (long)c * (taps - 1), span_pos[span] == 0, t,
+                    span_start[span]) + conv_b[c];
+  }
+  for (int i = nt * bs + tid; i < kGateTokens * bs; i += kRecThreads) us[i] = 0.f;
+  __syncthreads();
+  const float* wr = wr_t + (long)b * bs * bs;
+  const float* wi = wi_t + (long)b * bs * bs;
+  for (int o = tid; o < bs; o += kRecThreads) {
+    float ar[kGateTokens], ai[kGateTokens];
+#pragma unroll
+    for (int tt = 0; tt < kGateTokens; ++tt) ar[tt] = ai[tt] = 0.f;
+    for (int i = 0; i < bs; ++i) {
+      const float r = wr[(long)i * bs + o], g = wi[(long)i * bs + o];
+#pragma unroll
+      for (int tt = 0; tt < kGateTokens; ++tt) {
+        const float u = us[tt * bs + i];
+        ar[tt] = fmaf(r, u, ar[tt]);
+        ai[tt] = fmaf(g, u, ai[tt]);
+      }
+    }
+    const int c = b * bs + o;
+    const float rb = br[c], ib = bi[c], rt = rate[c];
+#pragma unroll
+    for (int tt = 0; tt < kGateTokens; ++tt) {
+      if (tt >= nt) break;
+      const float r = sigmoid_f32(ar[tt] + rb), ig = sigmoid_f32(ai[tt] + ib);
+      const float log_a = -rt * r;
+      const float a = expf(log_a);
+      const float mult = sqrtf(fmaxf(-expm1f(2.f * log_a), 0.f));      // sqrt(1 - a^2)
+      a_out[(tfirst + tt) * W + c] = a;
+      b_out[(tfirst + tt) * W + c] = mult * ig * us[tt * bs + o];
+    }
+  }
+}
+
+// S <- a S + b along a span, one thread a (span, channel); out = S * gelu_tanh(y + y_bias).  Eight
+// tokens' numbers are asked for at a time, so that the chain holds arithmetic only.
+template <typename T>
+__global__ __launch_bounds__(kRecThreads) void linear_recurrence_scan_kernel(
+    const float* __restrict__ a_in, const float* __restrict__ b_in, const float* __restrict__ proj, int nsplit,
+    long split_stride, const float* __restrict__ y_bias, float* __restrict__ state, long slot_stride,
+    const int* __restrict__ slots, const int* __restrict__ span_start, const int* __restrict__ span_pos,
+    T* __restrict__ out, int W) {
+  const int c = blockIdx.x * kRecThreads + threadIdx.x;
+  if (c >= W) return;
+  const int span = blockIdx.y;
+  const long t0 = span_start[span], t1 = span_start[span + 1];
+  float* st = state + (long)slots[span] * slot_stride + c;
+  float S = span_pos[span] == 0 ? 0.f : *st;
+  const float yb = y_bias[c];
+  constexpr int U = 8;
+  for (long tb = t0; tb < t1; tb += U) {
+    float a[U], b[U], y[U];
+#pragma unroll
+    for (int q = 0; q < U; ++q) {
+      const long t = min(tb + q, t1 - 1);
+      a[q] = a_in[t * W + c];
+      b[q] = b_in[t * W + c];
+      float v = 0.f;
+      for (int s = 0; s < nsplit; ++s) v += proj[s * split_stride + t * 2 * W + c];
+      y[q] = gate_act(v + yb, ACT_GELU_TANH);
+    }
+#pragma unroll
+    for (int q = 0; q < U; ++q) {
+      if (tb + q >= t1) break;
+      S = fmaf(a[q], S, b[q]);
+      out[(tb + q) * W + c] = from_f32<T>(S * y[q]);
+    }
+  }
+  *st = S;
+}
+
+// out = sa * (sum of a's slices) + sb * (sum of b's slices), element by element.
+__global__ void scaled_sum_kernel(float* __restrict__ out, const float* __restrict__ a, int na, long stride_a, float sa,
+                                  const float* __restrict__ b, int nb, long stride_b, float sb, long count) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float va = 0.f, vb = 0.f;
+  for (int s = 0; s < na; ++s) va += a[i + s * stride_a];
+  for (int s = 0; s < nb; ++s) vb += b[i + s * stride_b];
+  out[i] = fmaf(sa, va, sb * vb);
+}
+
+}  // namespace kllm
+
+using namespace kllm;
+
+extern "C" int kllm_scaled_sum(float* out, const float* a, int na, long stride_a, float sa, const float* b, int nb,
+                               long stride_b, float sb, long count, hipStream_t stream) {
+  KLLM_REQUIRE(out && a && b && na >= 1 && nb >= 1 && count > 0, "scaled_sum: null pointer or bad sizes");
+  hipLaunchKernelGGL(scaled_sum_kernel, dim3(ceil_div(count, 256)), dim3(256), 0, stream, out, a, na, stride_a, sa, b, nb,
+                     stride_b, sb, count);
+  KLLM_CHECK_LAUNCH("scaled_sum");
+  return 0;
+}
+
+extern "C" int kllm_conv_state_update(const float* proj, int nsplit, long split_stride, int cols, int col0, int C,
+                                      const float* in_bias, float* state, long slot_stride, int taps, const int* slots,
+                                      const int* span_start, const int* span_pos, int n_spans, hipStream_t stream) {
+  KLLM_REQUIRE(proj && state && slots && span_start && span_pos, "conv_state_update: null pointer");
+  KLLM_REQUIRE(nsplit >= 1 && cols > 0 && col0 >= 0 && C > 0 && col0 + C <= cols && n_spans > 0 && n_spans <= 65535,
+               "conv_state_update: bad sizes cols=%d col0=%d C=%d spans=%d", cols, col0, C, n_spans);
+  KLLM_REQUIRE(taps >= 1 && taps <= kMaxTaps, "conv_state_update: %d taps (1 to %d)", taps, kMaxTaps);
+  if (taps == 1) return 0;
+  hipLaunchKernelGGL(conv_state_update_kernel, dim3(ceil_div(C, kRecThreads), n_spans), dim3(kRecThreads), 0, stream,
+                     proj, nsplit, split_stride, (long)cols, col0, C, in_bias ? in_bias - col0 : nullptr, state,
+                     slot_stride, taps, slots, span_start, span_pos);
+  KLLM_CHECK_LAUNCH("conv_state_update");
+  return 0;
+}
+
+extern "C" int kllm_gated_delta_prep(const float* proj, int nsplit, long split_stride, const float* conv_w, int taps,
+                                     const float* state, long slot_stride, const float* a_log, const float* dt_bias,
+                                     const int* span_of_token, const int* slots, const int* span_start,
+                                     const int* span_pos, float* qn, float* kn, float* vv, float* gb, float* gate,
+                                     int n, int H, int G, int dk, int dv, float unit_eps, hipStream_t stream) {
+  KLLM_REQUIRE(proj && conv_w && state && a_log && dt_bias && span_of_token && slots && span_start && span_pos && qn &&
+                   kn && vv && gb && gate, "gated_delta_prep: null pointer");
+  KLLM_REQUIRE(n > 0 && H > 0 && G > 0 && H % G == 0 && dk > 0 && dv > 0 && nsplit >= 1,
+               "gated_delta_prep: bad sizes n=%d H=%d G=%d dk=%d dv=%d", n, H, G, dk, dv);
+  KLLM_REQUIRE(taps >= 1 && taps <= kMaxTaps, "gated_delta_prep: %d taps (1 to %d)", taps, kMaxTaps);
+  const size_t lds = ((size_t)2 * G * dk + (size_t)H * dv) * sizeof(float);
+  KLLM_REQUIRE(lds <= 64 * 1024, "gated_delta_prep: %zu bytes of a token's channels do not fit into LDS", lds);
+  hipLaunchKernelGGL(gated_delta_prep_kernel, dim3(n), dim3(kRecThreads), lds, stream, proj, nsplit, split_stride,
+                     conv_w, taps, state, slot_stride, a_log, dt_bias, span_of_token, slots, span_start, span_pos, qn,
+                     kn, vv, gb, gate, H, G, dk, dv, unit_eps);
+  KLLM_CHECK_LAUNCH("gated_delta_prep");
+  return 0;
+}
+
+extern "C" int kllm_gated_delta_max_dim(void) { return 16 * kDeltaParts; }
+
+extern "C" int kllm_gated_delta_scan(const float* qn, const float* kn, const float* vv, const float* gb, float* o_out,
+                                     float* state, long slot_stride, const int* slots, const int* span_start,
+                                     const int* span_pos, int n_spans, int H, int G, int dk, int dv,
+                                     hipStream_t stream) {
+  KLLM_REQUIRE(qn && kn && vv && gb && o_out && state && slots && span_start && span_pos,
+               "gated_delta_scan: null pointer");
+  KLLM_REQUIRE(n_spans > 0 && H > 0 && H <= 65535 && G > 0 && H % G == 0 && dk > 0 && dk <= 16 * kDeltaParts && dv > 0,
+               "gated_delta_scan: bad sizes spans=%d H=%d G=%d dk=%d dv=%d (keys of up to %d)", n_spans, H, G, dk, dv,
+               16 * kDeltaParts);
+  const dim3 grid(n_spans, H, ceil_div(dv, kDeltaCols));
+  KLLM_REQUIRE(grid.z <= 65535, "gated_delta_scan: values too wide for the grid");
+  const size_t lds = ((size_t)kDeltaBlock * (2 * dk + kDeltaCols + 2)) * sizeof(float);
+  const int nr = ceil_div(dk, kDeltaParts);
+#define KLLM_GDS(NR)                                                                                              \
+  hipLaunchKernelGGL(gated_delta_scan_kernel<NR>, grid, dim3(kRecThreads), lds, stream, qn, kn, vv, gb, o_out, \
+                     state, slot_stride, slots, span_start, span_pos, H, G, dk, dv)
+  if (nr <= 1) KLLM_GDS(1);
+  else if (nr <= 2) KLLM_GDS(2);
+  else if (nr <= 4) KLLM_GDS(4);
+  else if (nr <= 8) KLLM_GDS(8);
+  else KLLM_GDS(16);
+#undef KLLM_GDS
+  KLLM_CHECK_LAUNCH("gated_delta_scan");
+  return 0;
+}
+
+extern "C" int kllm_linear_recurrence_prep(const float* proj, int nsplit, long split_stride, const float* x_bias,
+                                           const float* conv_w, const float* conv_b, int taps, const float* state,
+                                           long slot_stride, const float* wr_t, const float* wi_t, const float* br,
+                                           const float* bi, const float* rate, const int* span_of_token,
+                                           const int* slots, const int* span_start, const int* span_pos, float* a_out,
+                                           float* b_out, int n, int W, int blocks, hipStream_t stream) {
+  KLLM_REQUIRE(proj && x_bias && conv_w && conv_b && state && wr_t && wi_t && br && bi && rate && span_of_token &&
+                   slots && span_start && span_pos && a_out && b_out, "linear_recurrence_prep: null pointer");
+  KLLM_REQUIRE(n > 0 && W > 0 && blocks > 0 && blocks <= 65535 && W % blocks == 0 && nsplit >= 1,
+               "linear_recurrence_prep: bad sizes n=%d W=%d blocks=%d", n, W, blocks);
+  KLLM_REQUIRE(taps >= 1 && taps <= kMaxTaps, "linear_recurrence_prep: %d taps (1 to %d)", taps, kMaxTaps);
+  const int bs = W / blocks;
+  const size_t lds = (size_t)kGateTokens * bs * sizeof(float);
+  KLLM_REQUIRE(lds <= 64 * 1024, "linear_recurrence_prep: blocks of %d channels do not fit into LDS", bs);
+  hipLaunchKernelGGL(linear_recurrence_prep_kernel, dim3(ceil_div(n, kGateTokens), blocks), dim3(kRecThreads), lds,
+                     stream, proj, nsplit, split_stride, x_bias, conv_w, conv_b, taps, state, slot_stride, wr_t, wi_t,
+                     br, bi, rate, span_of_token, slots, span_start, span_pos, a_out, b_out, n, W, bs);
+  KLLM_CHECK_LAUNCH("linear_recurrence_prep");
+  return 0;
+}
+
+extern "C" int kllm_linear_recurrence_scan(const float* a_in, const float* b_in, const float* proj, int nsplit,
+                                           long split_stride, const float* y_bias, float* state, long slot_stride,
+                                           const int* slots, const int* span_start, const int* span_pos, void* out,
+                                           int n_spans, int W, int dtype, hipStream_t stream) {
+  KLLM_REQUIRE(a_in && b_in && proj && y_bias && state && slots && span_start && span_pos && out,
+               "linear_recurrence_scan: null pointer");
+  KLLM_REQUIRE(n_spans > 0 && n_spans <= 65535 && W > 0 && nsplit >= 1, "linear_recurrence_scan: bad sizes spans=%d W=%d",
+               n_spans, W);
+  KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "linear_recurrence_scan: unknown dtype %d", dtype);
+  const dim3 grid(ceil_div(W, kRecThreads), n_spans);
+  if (dtype == DT_F32)
+    hipLaunchKernelGGL(linear_recurrence_scan_kernel<float>, grid, dim3(kRecThreads), 0, stream, a_in, b_in, proj,
+                       nsplit, split_stride, y_bias, state, slot_stride, slots, span_start, span_pos, (float*)out, W);
+  else
+    hipLaunchKernelGGL(linear_recurrence_scan_kernel<bf16_t>, grid, dim3(kRecThreads), 0, stream, a_in, b_in, proj,
+                       nsplit, split_stride, y_bias, state, slot_stride, slots, span_start, span_pos, (bf16_t*)out, W);
+  KLLM_CHECK_LAUNCH("linear_recurrence_scan");
+  return 0;
+}

@@ -169,7 +169,7 @@ __global__ __launch_bounds__(256) void qkv_norm_append_kernel(
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, int interleaved, int unit_norm,
     float eps, T* __restrict__ q_out, T* __restrict__ cache, const int* __restrict__ positions,
     const int* __restrict__ span_of_token, const int* __restrict__ block_table, int max_pages, int page_size,
-    int H, int KV, int dk, int dv) {
+    int H, int KV, int dk, int dv, const float* __restrict__ q_weight, const float* __restrict__ k_weight) {
   const long t = blockIdx.x;
   const int lane = threadIdx.x % kWave;
   const int item = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
@@ -229,16 +229,35 @@ __global__ __launch_bounds__(256) void qkv_norm_append_kernel(
       b[r] += src[eb[r]];
     }
   }
+  if (bias) {
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      if (lane + kWave * r >= pairs) continue;
+      a[r] += bias[base + ea[r]];
+      b[r] += bias[base + eb[r]];
+    }
+  }
+  const float* nw = is_q ? q_weight : k_weight;
+  if (nw) {     // a norm with weights in front of the rotation
+    float s0 = 0.f;
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+      if (lane + kWave * r < pairs) s0 += a[r] * a[r] + b[r] * b[r];
+    const float rs = 1.f / sqrtf(wave_sum(s0) / (float)dk + eps);
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      if (lane + kWave * r >= pairs) continue;
+      a[r] = a[r] * rs * nw[ea[r]];
+      b[r] = b[r] * rs * nw[eb[r]];
+    }
+    unit_norm = 0;
+  }
   float ss = 0.f;
 #pragma unroll
   for (int r = 0; r < 2; ++r) {
     const int j = lane + kWave * r;
     ra[r] = rb[r] = 0.f;
     if (j >= pairs) continue;
-    if (bias) {
-      a[r] += bias[base + ea[r]];
-      b[r] += bias[base + eb[r]];
-    }
     const bool turns = cos_t && j < rhalf;
     const float c = turns ? cos_t[t * rhalf + j] : 1.f, sn = turns ? sin_t[t * rhalf + j] : 0.f;
     ra[r] = a[r] * c - b[r] * sn;
@@ -329,8 +348,10 @@ extern "C" int kllm_qkv_norm_append(const float* qkv, int nsplit, long split_str
                                     const float* cos_t, const float* sin_t, int rot, int interleaved, int unit_norm,
                                     float eps, void* q_out, void* cache, const int* positions,
                                     const int* span_of_token, const int* block_table, int max_pages, int page_size,
-                                    int n, int H, int KV, int dk, int dv, int dtype, hipStream_t stream) {
+                                    int n, int H, int KV, int dk, int dv, int dtype, const float* q_weight,
+                                    const float* k_weight, hipStream_t stream) {
   KLLM_REQUIRE(qkv && q_out && cache && positions && span_of_token && block_table, "qkv_norm_append: null pointer");
+  KLLM_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), "qkv_norm_append: the two norm weights go together");
   KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && nsplit >= 1, "qkv_norm_append: bad sizes n=%d H=%d KV=%d nsplit=%d", n, H, KV,
                nsplit);
   KLLM_REQUIRE(dk > 0 && dk % 2 == 0 && dk <= 256 && dv > 0 && dv <= 256,
@@ -344,11 +365,11 @@ extern "C" int kllm_qkv_norm_append(const float* qkv, int nsplit, long split_str
   if (dtype == DT_F32)
     hipLaunchKernelGGL(qkv_norm_append_kernel<float>, grid, dim3(256), 0, stream, qkv, nsplit, split_stride, bias, cos_t,
                        sin_t, rot, interleaved, unit_norm, eps, (float*)q_out, (float*)cache, positions, span_of_token,
-                       block_table, max_pages, page_size, H, KV, dk, dv);
+                       block_table, max_pages, page_size, H, KV, dk, dv, q_weight, k_weight);
   else
     hipLaunchKernelGGL(qkv_norm_append_kernel<bf16_t>, grid, dim3(256), 0, stream, qkv, nsplit, split_stride, bias, cos_t,
                        sin_t, rot, interleaved, unit_norm, eps, (bf16_t*)q_out, (bf16_t*)cache, positions, span_of_token,
-                       block_table, max_pages, page_size, H, KV, dk, dv);
+                       block_table, max_pages, page_size, H, KV, dk, dv, q_weight, k_weight);
   KLLM_CHECK_LAUNCH("qkv_norm_append");
   return 0;
 }

@@ -33,6 +33,12 @@ _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bf
            "bf16": torch.bfloat16}
 
 
+def _entries(run):
+    """The (group, entry, writes) triples of one run of the cache plan: none, one, or one for each
+    need of a mixer that is made of several."""
+    return [] if run is None else list(run) if isinstance(run, list) else [run]
+
+
 def _numel(shape) -> int:
     n = 1
     for d in shape:
@@ -222,7 +228,7 @@ class Engine:
         for g, gp in paged:
             want[g] = asked
             if gp.need.window > 0 and self.max_model_len:
-                per_request = window_pages(self.max_model_len, step, o.page_size, gp.need.window)
+                per_request = window_pages(self.max_model_len, step, o.page_size, gp.need.window, gp.need.keep_first)
                 want[g] = min(asked, o.max_requests * per_request)
         if o.memory_bytes is not None and paged:
             budget = int(o.memory_bytes) - state_bytes
@@ -243,7 +249,7 @@ class Engine:
             need = gp.need
             if need.kind == "paged":
                 self._paged_group_of[g] = len(groups)
-                groups.append(GroupSpec(f"group{g}", o.page_size, want[g], need.window))
+                groups.append(GroupSpec(f"group{g}", o.page_size, want[g], need.window, need.keep_first if need.window else 0))
                 if need.value_width == need.head_dim:
                     shape = (2, need.kv_heads, o.page_size * need.head_dim)
                 else:       # keys and values of different widths (or no values): the mixer lays a page out
@@ -254,6 +260,7 @@ class Engine:
                     f"group{g}: {gp.entries} layers, {need.kv_heads} KV heads of {need.head_dim}"
                     + (f" (values of {need.value_width})" if need.value_width != need.head_dim else "")
                     + (f", window {need.window}" if need.window else "")
+                    + (f" and the first {need.keep_first}" if need.window and need.keep_first else "")
                     + f": {want[g]} pages of {o.page_size} tokens = {want[g] * o.page_size} tokens, "
                     f"{want[g] * page_bytes[g] / 2**20:.1f} MiB"
                     + (f" (asked for {asked} pages)" if want[g] != asked else ""))
@@ -280,9 +287,9 @@ class Engine:
             if gp.need.kind != "paged":
                 continue
             per_token = gp.need.kv_heads * (gp.need.head_dim + gp.need.value_width) * self.kv[g].element_size()
-            readers = sum(1 for r in self.model.cache_plan.runs if r is not None and r[0] == g)
+            readers = sum(1 for r in self.model.cache_plan.runs for e in _entries(r) if e[0] == g)
             for c in contexts:
-                total += readers * per_token * (min(c, gp.need.window) if gp.need.window else c)
+                total += readers * per_token * (min(c, gp.need.window + gp.need.keep_first) if gp.need.window else c)
         return total
 
     def step_read_bytes(self, contexts: Sequence[int]) -> int:
@@ -571,17 +578,21 @@ class Engine:
         return self.sample(logits, temperatures, uniforms)
 
     def _cache_views(self, ctx: StepContext):
+        def view(entry):
+            g, e, writes = entry
+            if g in self.kv:
+                return PagedCacheView(self.kv[g][e], ctx.block_tables[self._paged_group_of[g]],
+                                      self.options.page_size, writes)
+            return StateCacheView(self.state[g][e], ctx.slots, writes)
+
         views = []
         for entry in self.model.cache_plan.runs:
             if entry is None:
                 views.append(None)
-                continue
-            g, e, writes = entry
-            if g in self.kv:
-                views.append(PagedCacheView(self.kv[g][e], ctx.block_tables[self._paged_group_of[g]],
-                                            self.options.page_size, writes))
+            elif isinstance(entry, list):        # a mixer made of several: one view for each of its needs
+                views.append(tuple(view(e) for e in entry))
             else:
-                views.append(StateCacheView(self.state[g][e], ctx.slots, writes))
+                views.append(view(entry))
         return views
 
     # ------------------------------------------------------------------ sampling

@@ -29,8 +29,9 @@ class CacheGroupPlan:
 @dataclass
 class CachePlan:
     groups: List[CacheGroupPlan] = field(default_factory=list)
-    # per run of the schedule: (group, entry, writes) or None for a mixer without cache
-    runs: List[Optional[Tuple[int, int, bool]]] = field(default_factory=list)
+    # per run of the schedule: (group, entry, writes), None for a mixer without cache, or a list
+    # of such triples for a mixer made of several (one for each of its needs, in their order)
+    runs: List[object] = field(default_factory=list)
 
 
 class Model:
@@ -59,6 +60,21 @@ class Model:
                 raise ValueError(f"schedule entry {i} names layer {run.layer}, the model has "
                                  f"{len(self.blocks)}")
             need = self.blocks[run.layer].cache_need()
+            if isinstance(need, (list, tuple)):
+                # a mixer made of several: every need gets an entry of its own in its group
+                if run.cache_of is not None:
+                    raise ValueError(f"schedule entry {i}: a mixer with several caches shares none")
+                entries = []
+                for one in need:
+                    key = one.group_key()
+                    if key not in keys:
+                        keys[key] = len(plan.groups)
+                        plan.groups.append(CacheGroupPlan(one))
+                    g = keys[key]
+                    entries.append((g, plan.groups[g].entries, True))
+                    plan.groups[g].entries += 1
+                plan.runs.append(entries)
+                continue
             if need is None:
                 if run.cache_of is not None:
                     raise ValueError(f"schedule entry {i}: its mixer keeps no cache to share")
@@ -66,7 +82,7 @@ class Model:
                 continue
             if run.cache_of is not None:
                 j = run.cache_of
-                if not 0 <= j < i or plan.runs[j] is None or not plan.runs[j][2]:
+                if not 0 <= j < i or plan.runs[j] is None or isinstance(plan.runs[j], list) or not plan.runs[j][2]:
                     raise ValueError(
                         f"schedule entry {i} reads the cache of entry {j}, which must be an "
                         f"earlier entry that writes one")

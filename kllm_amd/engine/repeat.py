@@ -120,10 +120,15 @@ class _Names:
         return None
 
 
-def _view_tensors(view) -> Dict[tuple, torch.Tensor]:
+def _view_tensors(view, at=("c",)) -> Dict[tuple, torch.Tensor]:
     if view is None:
         return {}
-    return {("c", k): v for k, v in vars(view).items() if isinstance(v, torch.Tensor) and v.numel()}
+    if isinstance(view, (list, tuple)):      # a mixer made of several: a view for each
+        out = {}
+        for j, v in enumerate(view):
+            out.update(_view_tensors(v, at + (j,)))
+        return out
+    return {at + (k,): v for k, v in vars(view).items() if isinstance(v, torch.Tensor) and v.numel()}
 
 
 class _Unnamed(Exception):
@@ -203,7 +208,8 @@ class LayerRepeater:
             takes = getattr(block, "takes_next_norm", False) and nxt is not None
             cache = model.cache_plan.runs[i]
             keys.append((alike[run.layer], alike[nxt] if takes else None,
-                         None if cache is None else (cache[0], cache[2])))
+                         None if cache is None else tuple((c[0], c[2]) for c in cache) if isinstance(cache, list)
+                         else (cache[0], cache[2])))
         count: Dict[Any, int] = {}
         for k in keys:
             count[k] = count.get(k, 0) + 1
@@ -385,7 +391,9 @@ class _StepRepeater:
         values = []
         for path in t.paths:
             if path[0] == "c":
-                tensor = getattr(view, path[1], None)
+                tensor = view
+                for step in path[1:]:            # (a mixer made of several: the view's index first)
+                    tensor = tensor[step] if isinstance(step, int) and isinstance(tensor, (list, tuple)) else getattr(tensor, step, None)
                 if not isinstance(tensor, torch.Tensor):
                     return False
                 values.append(tensor.data_ptr())

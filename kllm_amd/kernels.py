@@ -21,7 +21,7 @@ import torch
 DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
 GEMV_BEST_ROWS = 0         # rows up to which they beat the MFMA kernels in bfloat16: none (a step at 1.1B sizes, one token: 1.036 against 0.963 ms)
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 
 class KernelError(RuntimeError):
@@ -91,7 +91,7 @@ def _declare(lib):
     sigs = {
         "kllm_last_error": [c_char_p, I],
         "kllm_device_info": [I, c_char_p, I],
-        "kllm_embed": [P, P, P, P, P, I, I, I, I, P],
+        "kllm_embed": [P, P, P, P, P, I, I, I, I, F, P, P],
         "kllm_add_rmsnorm": [P, P, I, I, L, P, P, I, P, I, I, F, I, P],
         "kllm_rope_tables": [P, P, P, I, I, D, P],
         "kllm_rope_append": [P, I, I, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, P],
@@ -112,10 +112,10 @@ def _declare(lib):
         "kllm_command_nargs": [I],
         "kllm_run_commands": [P, L, P, P],
         "kllm_fused_linear_max_parts": [],
-        "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F, P, I, P],
+        "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F, P, I, I, P],
         "kllm_norm_residual": [P, P, I, L, P, P, P, I, I, I, F, P, P, I, P, P, I, I, P],
         "kllm_rope_tables_freq": [P, P, P, P, I, I, D, P],
-        "kllm_qkv_norm_append": [P, I, L, P, P, P, I, I, I, F, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
+        "kllm_qkv_norm_append": [P, I, L, P, P, P, I, I, I, F, P, P, P, P, P, I, I, I, I, I, I, I, I, P, P, P],
         "kllm_gate_bias": [P, I, L, P, P, I, I, I, I, F, F, P],
         "kllm_moe_tile_rows": [],
         "kllm_moe_route": [P, I, L, P, I, I, I, P, P, P],
@@ -148,6 +148,19 @@ def _declare(lib):
         "kllm_delta_scan_max_dim": [],
         "kllm_delta_scan": [P, P, P, P, P, P, I, I, I, I, P],
         "kllm_delta_out": [P, P, P, F, P, I, I, I, I, P],
+        "kllm_conv_state_update": [P, I, L, I, I, I, P, P, L, I, P, P, P, I, P],
+        "kllm_gated_delta_prep": [P, I, L, P, I, P, L, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, P],
+        "kllm_gated_delta_max_dim": [],
+        "kllm_gated_delta_scan": [P, P, P, P, P, P, L, P, P, P, I, I, I, I, I, P],
+        "kllm_linear_recurrence_prep": [P, I, L, P, P, P, I, P, L, P, P, P, P, P, P, P, P, P, P, P, I, I, I, P],
+        "kllm_linear_recurrence_scan": [P, P, P, I, L, P, P, L, P, P, P, P, I, I, I, P],
+        "kllm_scaled_sum": [P, P, I, L, F, P, I, L, F, L, P],
+        "kllm_latent_max_row": [],
+        "kllm_latent_kv_append": [P, I, L, P, F, P, P, P, P, P, P, I, I, I, I, I, I, L, P],
+        "kllm_latent_norm": [P, I, L, L, P, F, P, I, I, I, P],
+        "kllm_latent_query": [P, I, L, P, P, P, P, I, I, I, I, I, I, P],
+        "kllm_attn_latent": [P, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
+        "kllm_latent_out": [P, P, P, I, L, L, P, I, I, I, I, I, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -167,7 +180,10 @@ LAUNCHING = ("kllm_embed", "kllm_add_rmsnorm", "kllm_rope_tables", "kllm_rope_ap
              "kllm_attn_decode", "kllm_attn_prefill", "kllm_sample", "kllm_gemm_act", "kllm_add_sinusoid", "kllm_unary_act",
              "kllm_group_norm_add", "kllm_qk_norm_append", "kllm_delta_prep", "kllm_delta_scan", "kllm_delta_out",
              "kllm_norm_residual", "kllm_rope_tables_freq", "kllm_qkv_norm_append", "kllm_gate_bias", "kllm_moe_route",
-             "kllm_moe_plan", "kllm_moe_expert", "kllm_moe_expert_rows", "kllm_moe_combine")
+             "kllm_moe_plan", "kllm_moe_expert", "kllm_moe_expert_rows", "kllm_moe_combine",
+             "kllm_conv_state_update", "kllm_gated_delta_prep", "kllm_gated_delta_scan", "kllm_linear_recurrence_prep",
+             "kllm_linear_recurrence_scan", "kllm_latent_kv_append", "kllm_latent_norm", "kllm_latent_query", "kllm_attn_latent",
+             "kllm_latent_out", "kllm_scaled_sum")
 DYNAMIC_ARGS = {"kllm_attn_prefill": (18, 19)}     # arguments that may be a StepValue
 STRUCT_ARGS = {"kllm_gemv_plain": (7,), "kllm_gemv_swiglu": (8,), "kllm_gemv_rope_append": (17,),
                "kllm_fused_linear": (2,)}
@@ -541,10 +557,13 @@ def calibrate_mfma(dtype_code_, iters, sink) -> float:
     return flops.value
 
 
-def embed(out, table, ids, from_sampled=None, sampled=None):
-    """out [n, d] = table[ids]; where ``from_sampled[t] >= 0`` the id is
-    ``sampled[from_sampled[t]]``, a token id still on the device."""
+def embed(out, table, ids, from_sampled=None, sampled=None, scale=1.0, copy=None):
+    """out [n, d] = scale * table[ids]; where ``from_sampled[t] >= 0`` the id is
+    ``sampled[from_sampled[t]]``, a token id still on the device.  ``copy`` [n, d] in the
+    table's dtype receives the same rows."""
     n, d = out.shape
+    if copy is not None and (tuple(copy.shape) != (n, d) or copy.dtype != table.dtype):
+        raise KernelError("embed: the copy of the rows does not fit")
     if ids.numel() < n or table.shape[1] != d:
         raise KernelError(f"embed: out {tuple(out.shape)}, table {tuple(table.shape)}, "
                           f"{ids.numel()} ids do not fit")
@@ -553,7 +572,7 @@ def embed(out, table, ids, from_sampled=None, sampled=None):
     _launch("kllm_embed", "embed", _ptr(out, "embed out", torch.float32), _ptr(table, "embed table"),
         _ptr(ids, "embed ids", torch.int32), _ptr(from_sampled, "embed from", torch.int32, True),
         _ptr(sampled, "embed sampled", torch.int32, True), n, d, table.shape[0], dtype_code(table.dtype),
-        _stream())
+        float(scale), _ptr(copy, "embed copy", None, True), _stream())
 
 
 def add_rmsnorm(x, delta=None, weight=None, out=None, rows=None, eps=0.0, write_x=None):
@@ -1042,8 +1061,9 @@ def paged_cache_fits(cache, n_kv_heads, page_size, head_dim, value_dim):
 
 
 def attn_generic(q, out, cache, positions, span_of_token, block_table, page_size, n_heads,
-                 n_kv_heads, head_dim, window, scale, slopes=None, value_dim=None, chunk=0, sink=False):
-    """``slopes`` (here and in the other attention wrappers): float32 [heads] or None; slopes[h]
+                 n_kv_heads, head_dim, window, scale, slopes=None, value_dim=None, chunk=0, sink=False, keep_first=0):
+    """``keep_first`` > 0: the first keep_first positions of a request stay readable behind the
+    window.  ``slopes`` (here and in the other attention wrappers): float32 [heads] or None; slopes[h]
     times the distance from the query to the key is taken off head h's scaled scores.
     ``value_dim``: width of a value (default: the key's); ``chunk`` > 0: the query at position p
     reads no key before p - p % chunk; ``sink``: the softmax's denominator has one more term,
@@ -1062,7 +1082,7 @@ def attn_generic(q, out, cache, positions, span_of_token, block_table, page_size
         _ptr(span_of_token, "attn span_of_token", torch.int32),
         _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size, n,
         n_heads, n_kv_heads, head_dim, vd, int(window), int(chunk), int(bool(sink)), float(scale),
-        _slopes(slopes, n_heads, "attn_generic"), dtype_code(q.dtype), _stream())
+        _slopes(slopes, n_heads, "attn_generic"), dtype_code(q.dtype), int(keep_first), _stream())
 
 
 GENERIC_MAX_PAGE_SIZE = 256     # pages of the kernel that takes every size
@@ -1193,8 +1213,8 @@ def add_sinusoid(x, positions, base=10000.0):
             _ptr(positions, "add_sinusoid positions", torch.int32), n, d, float(base), _stream())
 
 
-ACT_XIELU, ACT_TANH = 2, 3
-UNARY_ACTIVATIONS = dict(ACTIVATIONS, xielu=ACT_XIELU, tanh=ACT_TANH)
+ACT_XIELU, ACT_TANH, ACT_RELU_SQ = 2, 3, 4
+UNARY_ACTIVATIONS = dict(ACTIVATIONS, xielu=ACT_XIELU, tanh=ACT_TANH, relu2=ACT_RELU_SQ)
 
 
 def _splits(t, n, cols, who):
@@ -1401,11 +1421,12 @@ def rope_tables_freq(cos, sin, positions, freq, factor=1.0):
 
 def qkv_norm_append(qkv, q_out, cache, positions, span_of_token, block_table, page_size, n_heads, n_kv_heads,
                     head_dim, value_dim, bias=None, cos=None, sin=None, rotary_dim=0, interleaved=True,
-                    unit_norm=True, eps=0.0):
+                    unit_norm=True, eps=0.0, q_weight=None, k_weight=None):
     """qkv: float32 sums [nsplit, n, (H + KV) * head_dim + KV * value_dim].  Adds ``bias``, rotates the
     first ``rotary_dim`` elements of every query and key head (cos, sin [n, rotary_dim / 2]),
     divides every query and key head by its root mean square (``unit_norm``), writes q_out and
-    appends keys and values to the pages."""
+    appends keys and values to the pages.  With ``q_weight`` and ``k_weight`` (float32 [head_dim], shared
+    by the heads) the norm stands in front of the rotation and has these weights."""
     n = q_out.shape[0]
     cols = (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim
     nsplit, stride = _splits(qkv, n, cols, "qkv_norm_append")
@@ -1418,6 +1439,9 @@ def qkv_norm_append(qkv, q_out, cache, positions, span_of_token, block_table, pa
     rot = int(rotary_dim) if cos is not None else 0
     if cos is not None and (tuple(cos.shape) != (n, rot // 2) or tuple(sin.shape) != tuple(cos.shape)):
         raise KernelError("qkv_norm_append: cos/sin shapes do not fit")
+    if (q_weight is None) != (k_weight is None) or (q_weight is not None and (q_weight.numel() != head_dim
+                                                                              or k_weight.numel() != head_dim)):
+        raise KernelError("qkv_norm_append: the norms' weights do not fit")
     F32 = torch.float32
     _launch("kllm_qkv_norm_append", "qkv_norm_append", _ptr(qkv, "qkv_norm_append qkv", F32), nsplit, stride,
             _ptr(bias, "qkv_norm_append bias", F32, True), _ptr(cos, "qkv_norm_append cos", F32, True),
@@ -1426,7 +1450,9 @@ def qkv_norm_append(qkv, q_out, cache, positions, span_of_token, block_table, pa
             _ptr(positions, "qkv_norm_append positions", torch.int32),
             _ptr(span_of_token, "qkv_norm_append span_of_token", torch.int32),
             _ptr(block_table, "qkv_norm_append block_table", torch.int32), block_table.shape[1], page_size, n,
-            n_heads, n_kv_heads, head_dim, value_dim, dtype_code(q_out.dtype), _stream())
+            n_heads, n_kv_heads, head_dim, value_dim, dtype_code(q_out.dtype),
+            _ptr(q_weight, "qkv_norm_append q weight", F32, True), _ptr(k_weight, "qkv_norm_append k weight", F32, True),
+            _stream())
 
 
 GATE_CLAMPED_SWISH = 4     # g' = min(g, limit), u' = clamp(u, -limit, limit): g' sigmoid(alpha g') (u' + 1)
@@ -1527,3 +1553,224 @@ def moe_combine(y, xin, idx, wgt, out, experts, shared=None):
             _ptr(idx, "moe_combine idx", torch.int32), _ptr(wgt, "moe_combine wgt", torch.float32),
             _ptr(shared, "moe_combine shared", torch.float32, True), ns, stride,
             _ptr(out, "moe_combine out", torch.float32), n, d, top, int(experts), dtype_code(xin.dtype), _stream())
+
+
+# ----------------------------------------------------------------------------- recurrent mixers with a short convolution
+
+def _field(state, offset, who):
+    """Address of a field of the per-slot state: ``state`` [slots, floats] float32, the field
+    ``offset`` floats into a slot.  Returns (address in slot 0, floats per slot)."""
+    if state.dim() != 2 or state.dtype != torch.float32 or not 0 <= offset < state.shape[1]:
+        raise KernelError(f"{who}: state {tuple(state.shape)} {state.dtype}, field at {offset}")
+    return _ptr(state, who + " state", torch.float32) + 4 * int(offset), int(state.shape[1])
+
+
+def conv_state_update(proj, col0, channels, taps, state, offset, slots, span_start, span_pos, n_spans, in_bias=None):
+    """The convolution's field of the state ([channels, taps - 1] per slot, ``offset`` floats into
+    it) takes the inputs of every span's last taps - 1 positions: columns col0 .. col0 + channels
+    of the float32 sums ``proj`` [nsplit, n, cols] (plus ``in_bias`` [channels]); where a span is
+    shorter, the entries it had move up (zeros where the span starts at position 0)."""
+    n, cols = proj.shape[-2], proj.shape[-1]
+    nsplit, stride = _splits(proj, n, cols, "conv_state_update")
+    if taps <= 1:
+        return
+    addr, per_slot = _field(state, offset, "conv_state_update")
+    if (offset + channels * (taps - 1) > per_slot or col0 + channels > cols or slots.numel() < n_spans
+            or span_start.numel() < n_spans + 1 or (in_bias is not None and in_bias.numel() != channels)):
+        raise KernelError("conv_state_update: sizes do not fit")
+    I32 = torch.int32
+    _launch("kllm_conv_state_update", "conv_state_update", _ptr(proj, "conv proj", torch.float32), nsplit, stride, cols,
+            int(col0), int(channels), _ptr(in_bias, "conv bias", torch.float32, True), addr, per_slot, int(taps),
+            _ptr(slots, "conv slots", I32), _ptr(span_start, "conv span_start", I32), _ptr(span_pos, "conv span_pos", I32),
+            int(n_spans), _stream())
+
+
+def gated_delta_max_dim() -> int:
+    return limit("gated_delta_max_dim")
+
+
+def gated_delta_prep(proj, conv_w, taps, state, conv_offset, a_log, dt_bias, span_of_token, slots, span_start, span_pos,
+                     qn, kn, vv, gb, gate, heads, kv_heads, dim, vdim, unit_eps=1e-6):
+    """proj: float32 sums [nsplit, n, 2 G dk + 2 H dv + 2 H] of q | k | v | b | a | gate.  Convolution
+    (conv_w [2 G dk + H dv, taps], its earlier inputs from the state's field at ``conv_offset``) and
+    SiLU of q, k, v; q and k to unit vectors per head, q times dk^-1/2; gb [n, 2, H] = (exp(-exp(a_log)
+    softplus(a + dt_bias)), sigmoid(b)); gate [n, H dv] = silu of the gate's sums."""
+    n = qn.shape[0]
+    QK, HV = kv_heads * dim, heads * vdim
+    C = 2 * QK + HV
+    nsplit, stride = _splits(proj, n, C + 2 * heads + HV, "gated_delta_prep")
+    addr, per_slot = _field(state, conv_offset, "gated_delta_prep")
+    F32, I32 = torch.float32, torch.int32
+    if (tuple(conv_w.shape) != (C, taps) or a_log.numel() != heads or dt_bias.numel() != heads
+            or tuple(qn.shape) != (n, QK) or tuple(kn.shape) != (n, QK) or tuple(vv.shape) != (n, HV)
+            or tuple(gb.shape) != (n, 2, heads) or tuple(gate.shape) != (n, HV)
+            or conv_offset + C * (taps - 1) > per_slot or span_of_token.numel() < n):
+        raise KernelError("gated_delta_prep: shapes do not fit")
+    _launch("kllm_gated_delta_prep", "gated_delta_prep", _ptr(proj, "gated_delta proj", F32), nsplit, stride,
+            _ptr(conv_w, "gated_delta conv", F32), int(taps), addr, per_slot, _ptr(a_log, "gated_delta A", F32),
+            _ptr(dt_bias, "gated_delta dt", F32), _ptr(span_of_token, "gated_delta span_of_token", I32),
+            _ptr(slots, "gated_delta slots", I32), _ptr(span_start, "gated_delta span_start", I32),
+            _ptr(span_pos, "gated_delta span_pos", I32), _ptr(qn, "gated_delta qn", F32), _ptr(kn, "gated_delta kn", F32),
+            _ptr(vv, "gated_delta v", F32), _ptr(gb, "gated_delta gb", F32), _ptr(gate, "gated_delta gate", F32), n,
+            int(heads), int(kv_heads), int(dim), int(vdim), float(unit_eps), _stream())
+
+
+def gated_delta_scan(qn, kn, vv, gb, o_out, state, offset, slots, span_start, span_pos, n_spans, heads, kv_heads, dim,
+                     vdim):
+    """S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, each request through its state
+    ([heads, dim, vdim] float32 at ``offset`` floats into its slot; zero where a span's position is 0)."""
+    n = qn.shape[0]
+    addr, per_slot = _field(state, offset, "gated_delta_scan")
+    if (tuple(o_out.shape) != (n, heads * vdim) or tuple(vv.shape) != (n, heads * vdim)
+            or tuple(qn.shape) != (n, kv_heads * dim) or tuple(kn.shape) != tuple(qn.shape)
+            or tuple(gb.shape) != (n, 2, heads) or offset + heads * dim * vdim > per_slot
+            or slots.numel() < n_spans or span_start.numel() < n_spans + 1 or span_pos.numel() < n_spans):
+        raise KernelError("gated_delta_scan: shapes do not fit")
+    F32, I32 = torch.float32, torch.int32
+    _launch("kllm_gated_delta_scan", "gated_delta_scan", _ptr(qn, "gated_delta qn", F32), _ptr(kn, "gated_delta kn", F32),
+            _ptr(vv, "gated_delta v", F32), _ptr(gb, "gated_delta gb", F32), _ptr(o_out, "gated_delta o", F32), addr,
+            per_slot, _ptr(slots, "gated_delta slots", I32), _ptr(span_start, "gated_delta span_start", I32),
+            _ptr(span_pos, "gated_delta span_pos", I32), int(n_spans), int(heads), int(kv_heads), int(dim), int(vdim),
+            _stream())
+
+
+def linear_recurrence_prep(proj, x_bias, conv_w, conv_b, taps, state, conv_offset, wr_t, wi_t, br, bi, rate,
+                           span_of_token, slots, span_start, span_pos, a_out, b_out, blocks):
+    """proj: float32 sums [nsplit, n, 2 W] of y | x.  u = conv(x + x_bias) + conv_b; gates r, i =
+    sigmoid(block-diagonal products of u + biases), the matrices given [blocks, in, out]; a_out =
+    exp(-rate r), b_out = sqrt(1 - a^2) i u, both [n, W]."""
+    n, W = a_out.shape
+    nsplit, stride = _splits(proj, n, 2 * W, "linear_recurrence_prep")
+    addr, per_slot = _field(state, conv_offset, "linear_recurrence_prep")
+    bs = W // blocks
+    F32, I32 = torch.float32, torch.int32
+    if (W % blocks or tuple(wr_t.shape) != (blocks, bs, bs) or tuple(wi_t.shape) != (blocks, bs, bs)
+            or tuple(conv_w.shape) != (W, taps) or any(t.numel() != W for t in (x_bias, conv_b, br, bi, rate))
+            or tuple(b_out.shape) != (n, W) or conv_offset + W * (taps - 1) > per_slot or span_of_token.numel() < n):
+        raise KernelError("linear_recurrence_prep: shapes do not fit")
+    _launch("kllm_linear_recurrence_prep", "linear_recurrence_prep", _ptr(proj, "recurrence proj", F32), nsplit, stride,
+            _ptr(x_bias, "recurrence x bias", F32), _ptr(conv_w, "recurrence conv", F32),
+            _ptr(conv_b, "recurrence conv bias", F32), int(taps), addr, per_slot, _ptr(wr_t, "recurrence gate r", F32),
+            _ptr(wi_t, "recurrence gate i", F32), _ptr(br, "recurrence gate r bias", F32),
+            _ptr(bi, "recurrence gate i bias", F32), _ptr(rate, "recurrence rate", F32),
+            _ptr(span_of_token, "recurrence span_of_token", I32), _ptr(slots, "recurrence slots", I32),
+            _ptr(span_start, "recurrence span_start", I32), _ptr(span_pos, "recurrence span_pos", I32),
+            _ptr(a_out, "recurrence a", F32), _ptr(b_out, "recurrence b", F32), n, W, int(blocks), _stream())
+
+
+def linear_recurrence_scan(a_in, b_in, proj, y_bias, state, offset, slots, span_start, span_pos, n_spans, out):
+    """S <- a S + b along every span (state [W] float32 at ``offset`` floats into the slot); out
+    [n, W] = S * gelu_tanh(y + y_bias), y the first W columns of the sums ``proj`` [nsplit, n, 2 W]."""
+    n, W = a_in.shape
+    nsplit, stride = _splits(proj, n, 2 * W, "linear_recurrence_scan")
+    addr, per_slot = _field(state, offset, "linear_recurrence_scan")
+    if (tuple(b_in.shape) != (n, W) or tuple(out.shape) != (n, W) or y_bias.numel() != W or offset + W > per_slot
+            or slots.numel() < n_spans or span_start.numel() < n_spans + 1 or span_pos.numel() < n_spans):
+        raise KernelError("linear_recurrence_scan: shapes do not fit")
+    F32, I32 = torch.float32, torch.int32
+    _launch("kllm_linear_recurrence_scan", "linear_recurrence_scan", _ptr(a_in, "recurrence a", F32),
+            _ptr(b_in, "recurrence b", F32), _ptr(proj, "recurrence proj", F32), nsplit, stride,
+            _ptr(y_bias, "recurrence y bias", F32), addr, per_slot, _ptr(slots, "recurrence slots", I32),
+            _ptr(span_start, "recurrence span_start", I32), _ptr(span_pos, "recurrence span_pos", I32),
+            _ptr(out, "recurrence out"), int(n_spans), W, dtype_code(out.dtype), _stream())
+
+
+def scaled_sum(out, a, scale_a, b, scale_b):
+    """out [n, d] float32 = scale_a * a + scale_b * b; a and b are float32 sums [n, d] or [slices, n, d]."""
+    n, d = out.shape
+    na, sa = _splits(a, n, d, "scaled_sum")
+    nb, sb = _splits(b, n, d, "scaled_sum")
+    F32 = torch.float32
+    _launch("kllm_scaled_sum", "scaled_sum", _ptr(out, "scaled_sum out", F32), _ptr(a, "scaled_sum a", F32), na, sa,
+            float(scale_a), _ptr(b, "scaled_sum b", F32), nb, sb, float(scale_b), n * d, _stream())
+
+
+# ----------------------------------------------------------------------------- attention through low-rank latents
+
+def latent_max_row() -> int:
+    return limit("latent_max_row")
+
+
+def _columns(sums, first_column, width, who):
+    """(address, nsplit, slice stride, row stride) of ``width`` columns from ``first_column`` of float32
+    sums [n, cols] or [nsplit, n, cols]."""
+    n, cols = sums.shape[-2], sums.shape[-1]
+    nsplit, stride = _splits(sums, n, cols, who)
+    if first_column < 0 or first_column + width > cols:
+        raise KernelError(f"{who}: columns {first_column} .. {first_column + width} of {cols}")
+    return _ptr(sums, who + " sums", torch.float32) + 4 * int(first_column), nsplit, stride, cols
+
+
+def latent_kv_append(sums, first_column, weight, eps, cos, sin, cache, positions, span_of_token, block_table, page_size,
+                     rank, rot_dim):
+    """Columns first_column .. + rank + rot_dim of the float32 sums: the first ``rank`` through an RMS
+    norm with ``weight``, the rest rotated (halves paired; cos, sin [n, rot_dim / 2]); the row is
+    appended to the pages (``cache`` [pages, page_size * (rank + rot_dim)])."""
+    n = cos.shape[0]
+    row = rank + rot_dim
+    addr, nsplit, stride, cols = _columns(sums, first_column, row, "latent_kv_append")
+    if (sums.shape[-2] != n or cache.dim() != 2 or cache.shape[1] != page_size * row or weight.numel() != rank
+            or tuple(cos.shape) != (n, rot_dim // 2) or tuple(sin.shape) != tuple(cos.shape)
+            or positions.numel() < n or span_of_token.numel() < n):
+        raise KernelError("latent_kv_append: shapes do not fit")
+    F32, I32 = torch.float32, torch.int32
+    _launch("kllm_latent_kv_append", "latent_kv_append", addr, nsplit, stride,
+            _ptr(weight, "latent norm", F32), float(eps), _ptr(cos, "latent cos", F32), _ptr(sin, "latent sin", F32),
+            _ptr(cache, "latent cache"), _ptr(positions, "latent positions", I32),
+            _ptr(span_of_token, "latent span_of_token", I32), _ptr(block_table, "latent block_table", I32),
+            block_table.shape[1], int(page_size), n, int(rank), int(rot_dim), dtype_code(cache.dtype), cols, _stream())
+
+
+def latent_norm(sums, first_column, weight, eps, out):
+    """out [n, r] = RMS norm with ``weight`` of columns first_column .. + r of the float32 sums."""
+    n, r = out.shape
+    addr, nsplit, stride, cols = _columns(sums, first_column, r, "latent_norm")
+    if sums.shape[-2] != n or weight.numel() != r:
+        raise KernelError("latent_norm: shapes do not fit")
+    _launch("kllm_latent_norm", "latent_norm", addr, nsplit, stride, cols, _ptr(weight, "latent norm", torch.float32),
+            float(eps), _ptr(out, "latent_norm out"), n, r, dtype_code(out.dtype), _stream())
+
+
+def latent_query(q, w_uk, cos, sin, out, heads, dim, rot_dim, rank):
+    """q: float32 sums [nsplit, n, H (dim + rot_dim)], a head laid out [dim | rot_dim].  out [n, H
+    (rank + rot_dim)]: per head the first dim folded through w_uk ([H dim, rank]: sum_i q_i w[i, :]),
+    then the rotated rest."""
+    n = out.shape[0]
+    nsplit, stride = _splits(q, n, heads * (dim + rot_dim), "latent_query")
+    if (tuple(out.shape) != (n, heads * (rank + rot_dim)) or tuple(w_uk.shape) != (heads * dim, rank)
+            or w_uk.dtype != out.dtype or tuple(cos.shape) != (n, rot_dim // 2) or tuple(sin.shape) != tuple(cos.shape)):
+        raise KernelError("latent_query: shapes do not fit")
+    F32 = torch.float32
+    _launch("kllm_latent_query", "latent_query", _ptr(q, "latent q", F32), nsplit, stride, _ptr(w_uk, "latent w_uk"),
+            _ptr(cos, "latent cos", F32), _ptr(sin, "latent sin", F32), _ptr(out, "latent q out"), n, int(heads),
+            int(dim), int(rot_dim), int(rank), dtype_code(out.dtype), _stream())
+
+
+def attn_latent(q, out, cache, positions, span_of_token, block_table, page_size, heads, row, rank, scale):
+    """Causal attention of q [n, H row] over cached rows of ``row`` elements whose first ``rank``
+    are also the values: out [n, H rank]."""
+    n = q.shape[0]
+    if (tuple(q.shape) != (n, heads * row) or tuple(out.shape) != (n, heads * rank) or q.dtype != cache.dtype
+            or out.dtype != q.dtype or cache.dim() != 2 or cache.shape[1] != page_size * row
+            or positions.numel() < n or span_of_token.numel() < n):
+        raise KernelError("attn_latent: shapes or dtypes do not fit")
+    I32 = torch.int32
+    _launch("kllm_attn_latent", "attn_latent", _ptr(q, "attn_latent q"), _ptr(out, "attn_latent out"),
+            _ptr(cache, "attn_latent cache"), _ptr(positions, "attn_latent positions", I32),
+            _ptr(span_of_token, "attn_latent span_of_token", I32), _ptr(block_table, "attn_latent block_table", I32),
+            block_table.shape[1], int(page_size), n, int(heads), int(row), int(rank), float(scale), dtype_code(q.dtype),
+            _stream())
+
+
+def latent_out(attended, w_uv, out, heads, vdim, rank, gate=None, gate_column=0):
+    """out [n, H vdim] = per head w_uv ([H vdim, rank]) times attended [n, H rank], times sigmoid of
+    columns gate_column .. + H vdim of the float32 sums ``gate`` (None: no gate)."""
+    n = out.shape[0]
+    addr, nsplit, stride, cols = _columns(gate, gate_column, heads * vdim, "latent_out") if gate is not None else (0, 0, 0, 0)
+    if (tuple(attended.shape) != (n, heads * rank) or tuple(out.shape) != (n, heads * vdim)
+            or tuple(w_uv.shape) != (heads * vdim, rank) or w_uv.dtype != out.dtype or attended.dtype != out.dtype
+            or (gate is not None and gate.shape[-2] != n)):
+        raise KernelError("latent_out: shapes or dtypes do not fit")
+    _launch("kllm_latent_out", "latent_out", _ptr(attended, "latent attended"), _ptr(w_uv, "latent w_uv"),
+            addr, nsplit, stride, cols, _ptr(out, "latent out"), n, int(heads), int(vdim), int(rank),
+            dtype_code(out.dtype), _stream())

@@ -1,5 +1,6 @@
 from . import llama  # registers "LlamaForCausalLM"
 from . import nusilix  # registers "Nusilix"
 from . import ribovik  # registers "Ribovik"
+from . import natenex  # registers "Natenex"
 
-__all__ = ["llama", "nusilix", "ribovik"]
+__all__ = ["llama", "nusilix", "ribovik", "natenex"]

@@ -15,7 +15,8 @@ query to the key), ``chunk`` (0: none; c: a chunked mask, the query at position
 p reads no key before p - p % c, chunks counted from the request's position 0),
 ``sink`` (False; True: the softmax's denominator has one more term, exp(0): a
 key whose score is 0 and that has no value), ``value_dim`` (width of a value;
-default: the key's).
+default: the key's), ``keep_first`` (with a window: the first ``keep_first``
+positions of a request stay readable behind it, at their true positions).
 Tensors: ``<prefix>.{q,k,v,o}_proj.weight``.  The three input projections are
 kept as one matrix so that a step reads one weight for them.
 """
@@ -84,10 +85,13 @@ class CausalSelfAttention(Part):
         self.chunk = int(self.param("chunk", 0) or 0)
         self.sink = bool(self.param("sink", False))
         self.value_dim = int(self.param("value_dim", None) or self.head_dim)
-        if self.chunk < 0 or not 0 < self.value_dim <= 256:
-            raise ValueError(f"attention: chunk {self.chunk} or value_dim {self.value_dim} out of range")
+        self.keep_first = int(self.param("keep_first", 0) or 0) if self.window else 0
+        if self.chunk < 0 or self.keep_first < 0 or not 0 < self.value_dim <= 256:
+            raise ValueError(f"attention: chunk {self.chunk}, keep_first {self.keep_first} or value_dim "
+                             f"{self.value_dim} out of range")
         # layers with the same window and chunk read alike
-        self.step_values_key = f"attention.keys.window{self.window}" + (f".chunk{self.chunk}" if self.chunk else "")
+        self.step_values_key = (f"attention.keys.window{self.window}" + (f".chunk{self.chunk}" if self.chunk else "")
+                                + (f".first{self.keep_first}" if self.keep_first else ""))
         self.own_kv = bool(self.param("own_kv", True))
         if self.heads % self.kv_heads:
             raise ValueError(f"attention: {self.heads} heads are not a multiple of {self.kv_heads} KV heads")
@@ -146,7 +150,8 @@ class CausalSelfAttention(Part):
 
     def cache_need(self):
         return CacheNeed("paged", kv_heads=self.kv_heads, head_dim=self.head_dim, window=self.window,
-                         value_dim=self.value_dim if self.value_dim != self.head_dim else None)
+                         value_dim=self.value_dim if self.value_dim != self.head_dim else None,
+                         keep_first=self.keep_first)
 
     def flops(self, tokens, keys_read=0.0):
         # the projections, and per key read a score and a value product for every head
@@ -226,12 +231,14 @@ class CausalSelfAttention(Part):
             prompt_ok = self.head_dim in K.PREFILL_HEAD_DIMS
         else:
             fast = prompt_ok = K.attn_f32_fits(self.head_dim, cache.page_size)
-        # the kernels on the matrix cores take keys and values of one width
-        fast = fast and mode != "generic" and self.value_dim == self.head_dim and not self.FAST_KERNELS_OFF
+        # the kernels on the matrix cores take keys and values of one width, and one run of keys a query
+        fast = (fast and mode != "generic" and self.value_dim == self.head_dim and not self.FAST_KERNELS_OFF
+                and not self.keep_first)
         if not fast:
             K.attn_generic(q, out, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
                            cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,
-                           self.scale, slopes=self.slopes, value_dim=self.value_dim, chunk=self.chunk, sink=self.sink)
+                           self.scale, slopes=self.slopes, value_dim=self.value_dim, chunk=self.chunk, sink=self.sink,
+                           keep_first=self.keep_first)
             return
         n = q.shape[0]
         short = ctx.lists.get("attention.spans.short")
@@ -412,6 +419,65 @@ class UnitNormAttention(CausalSelfAttention):
         K.qkv_norm_append(qkv, q, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table, cache.page_size,
                           self.heads, self.kv_heads, self.head_dim, self.value_dim, bias=self.bias, cos=cos, sin=sin,
                           rotary_dim=self.rotary_dim, interleaved=self.interleaved, unit_norm=True, eps=self.eps)
+        out = ctx.buf("attn.out", (n, self.out_dim), dtype)
+        self.attend(ctx, q, out, cache)
+        return decode_linear(ctx, out, self.w_o, "attn.proj", self._tiled.get("o"))
+
+
+@register_part("mixer", "attention_qk_norm")
+class NormedQueryKeyAttention(CausalSelfAttention):
+    """Attention whose queries and keys pass an RMS norm per head, with a weight of the head's size
+    that all heads share, in front of the rotation: q = W_q h, k = W_k h, v = W_v h without biases;
+    every query and key head is divided by its root mean square and multiplied by the weight; the
+    first ``rotary_dim`` elements of every head then turn with the position (the position part
+    says how); the score is (q . k) * ``scale``; mask (``window``, ``keep_first``, ``chunk``),
+    ``sink`` and the kernels are the base class's; values may have a width of their own.
+
+    Parameters beyond the base class's: ``eps``.
+    Tensors: ``<prefix>.{q,k,v,o}.weight``, ``.{q,k}.norm``."""
+    takes_normed = False
+    fills_sink = False
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        if not self.own_kv:
+            raise ValueError("attention_qk_norm: keeps its own keys and values")
+        self.eps = float(self.param("eps"))
+        self.v_dim = self.kv_heads * self.value_dim
+        self.q_norm = self.k_norm = None
+
+    def weight_specs(self):
+        return [WeightSpec(self.tensor_name("q.weight"), (self.q_dim, self.hidden)),
+                WeightSpec(self.tensor_name("k.weight"), (self.kv_dim, self.hidden)),
+                WeightSpec(self.tensor_name("v.weight"), (self.v_dim, self.hidden)),
+                WeightSpec(self.tensor_name("o.weight"), (self.hidden, self.out_dim)),
+                WeightSpec(self.tensor_name("q.norm"), (self.head_dim,), "vector"),
+                WeightSpec(self.tensor_name("k.norm"), (self.head_dim,), "vector")]
+
+    def bind(self, weights):
+        self._bind_slopes()
+        self.w_in = torch.cat([weights[self.tensor_name(t + ".weight")] for t in ("q", "k", "v")], dim=0).contiguous()
+        self.w_o = weights[self.tensor_name("o.weight")]
+        self.q_norm = weights[self.tensor_name("q.norm")]
+        self.k_norm = weights[self.tensor_name("k.norm")]
+        # second copies for decode batches, in the order that kernel reads them
+        self._tiled = {"in": tiled_copy(self.runtime, self.w_in, K.LINEAR_PARTS),
+                       "o": tiled_copy(self.runtime, self.w_o, K.LINEAR_PARTS)}
+
+    def forward(self, ctx, xn, cache):
+        n = xn.shape[0]
+        dtype = self.runtime.dtype
+        if not cache.write:
+            raise ValueError("attention_qk_norm: the run writes its own cache")
+        qkv = decode_linear(ctx, xn, self.w_in, "attn.qkv", self._tiled.get("in"))
+        q = ctx.buf("attn.q", (n, self.q_dim), dtype)
+        cos = sin = None
+        if self.position is not None and hasattr(self.position, "tables"):
+            cos, sin = self.position.tables(ctx)
+        K.qkv_norm_append(qkv, q, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table, cache.page_size,
+                          self.heads, self.kv_heads, self.head_dim, self.value_dim, cos=cos, sin=sin,
+                          rotary_dim=self.rotary_dim, interleaved=self.interleaved, unit_norm=False, eps=self.eps,
+                          q_weight=self.q_norm, k_weight=self.k_norm)
         out = ctx.buf("attn.out", (n, self.out_dim), dtype)
         self.attend(ctx, q, out, cache)
         return decode_linear(ctx, out, self.w_o, "attn.proj", self._tiled.get("o"))

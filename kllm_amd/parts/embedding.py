@@ -1,7 +1,7 @@
 """Token embedding and output head.
 
 Embedding: x[t, :] = E[id_t, :], no scaling (backend/model.cu:89-95,
-:1056-1060).  Head: logits = xn . W^T in float32 for the wanted rows
+:1056-1060) unless a design asks for a constant factor (``scale``).  Head: logits = xn . W^T in float32 for the wanted rows
 (:1185-1188).  The head names its own tensor; a tied head simply names the
 embedding's table (the reference resolves tying offline by copying it:
 tools/convert_hf.py:81-82).
@@ -34,6 +34,8 @@ class TokenEmbedding(Part):
         eps = self.param("norm_eps", None)
         self.norm_eps = float(eps) if eps is not None else None
         self.norm_weight = None
+        # a constant on the embedded rows (the table itself stays as it is, for a head that shares it)
+        self.scale = float(self.param("scale", 1.0))
 
     def weight_specs(self):
         specs = [WeightSpec(self.tensor_name("weight"), (self.vocab, self.hidden))]
@@ -54,10 +56,15 @@ class TokenEmbedding(Part):
 
     def forward(self, ctx, token_ids):
         x = ctx.buf("x", (ctx.n, self.hidden), torch.float32)
+        # with ``stream_rows`` the rows are also left in the compute dtype, for a first sub-layer that
+        # reads the stream itself
+        copy = None
+        if self.param("stream_rows", False) and self.norm_eps is None and self.position is None:
+            copy = stream_copy(ctx, x, fill=False)
         if ctx.sampled is not None and ctx.token_from is not None:
-            K.embed(x, self.table, token_ids, ctx.token_from, ctx.sampled)
+            K.embed(x, self.table, token_ids, ctx.token_from, ctx.sampled, scale=self.scale, copy=copy)
         else:
-            K.embed(x, self.table, token_ids)
+            K.embed(x, self.table, token_ids, scale=self.scale, copy=copy)
         if self.norm_eps is not None:
             K.norm_residual(x, self.norm_weight, eps=self.norm_eps, out=stream_copy(ctx, x, fill=False))
         return x

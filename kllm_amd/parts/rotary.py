@@ -54,6 +54,8 @@ def scaled_frequencies(dims, base, scaling=None):
     freq = [float(base) ** (-2.0 * i / dims) for i in range(half)]
     if scaling is None:
         return freq, 1.0
+    if scaling[0] == "by_wavelength":
+        return wavelength_scaled(freq, *scaling[1:]), 1.0
     factor, original, fast, slow = (float(v) for v in scaling)
 
     def pair_of(turns):
@@ -68,6 +70,25 @@ def scaled_frequencies(dims, base, scaling=None):
     return out, 0.1 * math.log(factor) + 1.0
 
 
+def wavelength_scaled(freq, factor, low, high, original):
+    """Frequencies slowed down by their wavelength l = 2 pi / f: kept where l < original / high,
+    divided by ``factor`` where l > original / low, and between the two blended linearly in
+    s = (original / l - low) / (high - low): (1 - s) f / factor + s f.  All in double."""
+    import math
+    factor, low, high, original = float(factor), float(low), float(high), float(original)
+    out = []
+    for f in freq:
+        wavelength = 2.0 * math.pi / f
+        if wavelength < original / high:
+            out.append(f)
+        elif wavelength > original / low:
+            out.append(f / factor)
+        else:
+            s = (original / wavelength - low) / (high - low)
+            out.append((1.0 - s) * f / factor + s * f)
+    return out
+
+
 @register_part("position", "rotary_scaled")
 class ScaledRotaryEncoding(Part):
     """Rotation of the first ``rotary_dim`` elements of a head, neighbours paired ((2j, 2j + 1);
@@ -75,8 +96,9 @@ class ScaledRotaryEncoding(Part):
     ``scaled_frequencies``.  A mixer reads ``rotary_dim`` and ``interleaved`` and applies the
     tables; angles are taken in double and the tables rounded to float32 once.
 
-    Parameters: ``rotary_dim``, ``base``, ``scaling`` (None or (factor, original, fast, slow)),
-    ``interleaved`` (default True).  No tensors of the checkpoint."""
+    Parameters: ``rotary_dim``, ``base``, ``scaling`` (None, (factor, original, fast, slow) for the
+    stretch by pair index, or ("by_wavelength", factor, low, high, original) for the one of
+    ``wavelength_scaled``), ``interleaved`` (default True).  No tensors of the checkpoint."""
     graph_safe = True
     records_launches = True
 

@@ -34,7 +34,8 @@ class CacheNeed:
 
     kind "paged": keys and values per token, in pages; ``window`` > 0 means
     only the last ``window`` positions are ever read, so pages behind it are
-    given back.  A token's entry is, per KV head, a key of ``head_dim`` and a
+    given back; with ``keep_first`` > 0 the first ``keep_first`` positions of a
+    request stay readable too, and their pages are kept.  A token's entry is, per KV head, a key of ``head_dim`` and a
     value of ``value_dim`` elements (default: as wide as the key; 0: no value,
     one vector per token).  With equal widths a page is handed to the mixer as
     [2, kv_heads, page_size * head_dim]; otherwise as a flat run of
@@ -47,6 +48,7 @@ class CacheNeed:
     kv_heads: int = 0
     head_dim: int = 0
     window: int = 0
+    keep_first: int = 0
     state_shape: Tuple[int, ...] = ()
     value_dim: Optional[int] = None
     dtype: Optional[str] = None
@@ -57,7 +59,8 @@ class CacheNeed:
 
     def group_key(self):
         if self.kind == "paged":
-            return ("paged", self.kv_heads, self.head_dim, self.window, self.value_width, self.dtype)
+            return ("paged", self.kv_heads, self.head_dim, self.window, self.value_width, self.dtype,
+                    self.keep_first if self.window else 0)
         return ("state", self.dtype) + tuple(self.state_shape)
 
 
