@@ -3,8 +3,8 @@
 config.json names the architecture in ``architecture`` and gives ``vocab``, ``width``,
 ``embedding`` (``scale``), ``norm`` (``eps``) and ``layers``: per layer its ``type``, the sizes of
 its mixer (``mixer``), its feed-forward (``mlp``: null for none, or ``kind`` "dense" with ``ff``)
-and optionally ``weights_of``: the index of an earlier layer whose tensors this layer runs with
-(it keeps a cache or state of its own).
+and optionally ``weights_of``: the index of another layer whose tensors this layer runs with
+(it keeps a cache or state of its own, and the rest of its entry equals that layer's).
 
 Mixers by ``type``:
 
@@ -240,14 +240,17 @@ class NatenexConfig(ModelConfig):
             source = None
             if e.has("weights_of"):
                 source = e.get("weights_of")
-                if isinstance(source, bool) or not isinstance(source, int) or not 0 <= source < i:
-                    raise ConfigError(f"{at}: 'weights_of' must name an earlier layer, got {source!r}")
-                other = layers[source]
-                if other.weights_of is not None:
-                    raise ConfigError(f"{at}: 'weights_of' names layer {source}, which has no tensors of its own")
-                if (other.type, other.mixer, other.ff) != (kind, mixer, ff):
-                    raise ConfigError(f"{at}: a layer that runs with layer {source}'s tensors has its sizes")
+                if isinstance(source, bool) or not isinstance(source, int) or not 0 <= source < len(entries) or source == i:
+                    raise ConfigError(f"{at}: 'weights_of' must name another layer, got {source!r}")
             layers.append(NatenexLayer(kind, mixer, ff, source))
+        for i, layer in enumerate(layers):
+            if layer.weights_of is None:
+                continue
+            other, at = layers[layer.weights_of], f"{where}:layers[{i}]"
+            if other.weights_of is not None:
+                raise ConfigError(f"{at}: 'weights_of' names layer {layer.weights_of}, which has no tensors of its own")
+            if (other.type, other.mixer, other.ff) != (layer.type, layer.mixer, layer.ff):
+                raise ConfigError(f"{at}: a layer that runs with layer {layer.weights_of}'s tensors has its sizes")
         return cls(architecture="Natenex", vocab=vocab, width=width, layers=tuple(layers), norm_eps=eps,
                    embedding_scale=scale)
 

@@ -1560,7 +1560,7 @@ def moe_combine(y, xin, idx, wgt, out, experts, shared=None):
 def _field(state, offset, who):
     """Address of a field of the per-slot state: ``state`` [slots, floats] float32, the field
     ``offset`` floats into a slot.  Returns (address in slot 0, floats per slot)."""
-    if state.dim() != 2 or state.dtype != torch.float32 or not 0 <= offset < state.shape[1]:
+    if state.dim() != 2 or state.dtype != torch.float32 or not 0 <= offset <= state.shape[1]:
         raise KernelError(f"{who}: state {tuple(state.shape)} {state.dtype}, field at {offset}")
     return _ptr(state, who + " state", torch.float32) + 4 * int(offset), int(state.shape[1])
 

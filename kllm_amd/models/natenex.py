@@ -57,10 +57,14 @@ def build_natenex(cfg: NatenexConfig) -> ModelSpec:
         return PartSpec("linear_recurrence", p, hidden=d, width=r.width, blocks=r.blocks, taps=r.conv,
                         decay_scale=RECURRENCE_DECAY_SCALE, names=names)
 
-    layers, index_of, schedule = [], {}, []
+    # a layer that runs with another's tensors is that layer, listed once more in the running order
+    # (its own cache or state, no tensors)
+    own = [i for i, layer in enumerate(cfg.layers) if layer.weights_of is None]
+    index_of = {i: k for k, i in enumerate(own)}
+    schedule = [Run(index_of[i if layer.weights_of is None else layer.weights_of]) for i, layer in enumerate(cfg.layers)]
+    layers = []
     for i, layer in enumerate(cfg.layers):
-        if layer.weights_of is not None:         # the same layer once more: its own cache or state, no tensors
-            schedule.append(Run(index_of[layer.weights_of]))
+        if layer.weights_of is not None:
             continue
         p, m = f"l{i}.mix", layer.mixer
         if layer.type == "parallel":
@@ -83,8 +87,6 @@ def build_natenex(cfg: NatenexConfig) -> ModelSpec:
             f = f"l{i}.mlp"
             ff = PartSpec("dense_mlp", f, hidden=d, intermediate=layer.ff, activation="relu2",
                           names={"up.weight": f"{f}.up", "down.weight": f"{f}.down"})
-        index_of[i] = len(layers)
-        schedule.append(Run(len(layers)))
         layers.append(LayerSpec(mixer=mixer, feed_forward=ff, norm_mixer=norm(f"l{i}.norm1"),
                                 norm_feed_forward=norm(f"l{i}.norm2") if ff is not None else None,
                                 block="sublayer_norm"))

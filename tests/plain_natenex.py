@@ -233,3 +233,90 @@ def forward(cfg, w, tokens, taps=None):
         if taps is not None:
             taps.append(x.clone())
     return rms_norm(x, w["final.norm"], eps) @ w["embed"].T
+
+
+def greedy(cfg, w, prompt, steps):
+    """The ``steps`` tokens that follow ``prompt`` when the likeliest is taken each time."""
+    toks = list(prompt)
+    for _ in range(steps):
+        toks.append(int(torch.argmax(forward(cfg, w, toks)[-1])))
+    return toks[len(prompt):]
+
+
+# ----------------------------------------------------------------------------- token by token
+
+def linear_recurrence_step(x_t, state, conv_inputs, w, p, m):
+    """One token through the gated linear recurrence from (state [width], the last taps - 1
+    inputs of the convolution [taps - 1, width]); returns (output before W_o, state, inputs)."""
+    width, blocks = m["width"], m["blocks"]
+    y = gelu_tanh(w[p + ".y"] @ x_t + w[p + ".y.b"])
+    xin = w[p + ".x"] @ x_t + w[p + ".x.b"]
+    window = torch.cat([conv_inputs, xin[None]], dim=0)
+    u = (window.T * w[p + ".conv"]).sum(-1) + w[p + ".conv.b"]
+    ub = u.reshape(blocks, width // blocks)
+    r = torch.sigmoid(torch.einsum("bi,boi->bo", ub, w[p + ".ra"]) + w[p + ".ra.b"]).reshape(width)
+    i = torch.sigmoid(torch.einsum("bi,boi->bo", ub, w[p + ".ri"]) + w[p + ".ri.b"]).reshape(width)
+    a = torch.exp(-8.0 * r * softplus(w[p + ".lam"]))
+    state = a * state + torch.sqrt(1.0 - a * a) * i * u
+    return state * y, state, window[1:]
+
+
+# ----------------------------------------------------------------------------- random weights
+
+def _layer_tensors(layer, i, width, g):
+    def mat(o, k):
+        return torch.randn(o, k, generator=g, dtype=F64) / math.sqrt(k)
+
+    def vec(n, mean=1.0, spread=0.2):
+        return mean + spread * torch.randn(n, generator=g, dtype=F64)
+
+    out, p, m = {}, f"l{i}.mix", layer["mixer"]
+    out[f"l{i}.norm1"] = vec(width)
+    if layer["type"] == "parallel":
+        a, r = m["left"], m["right"]
+        q = p + ".left"
+        out[q + ".q"], out[q + ".k"] = mat(a["heads"] * a["dim"], width), mat(a["kv_heads"] * a["dim"], width)
+        out[q + ".v"], out[q + ".o"] = mat(a["kv_heads"] * a["vdim"], width), mat(width, a["heads"] * a["vdim"])
+        out[q + ".q.norm"], out[q + ".k.norm"] = vec(a["dim"], 1.5, 0.4), vec(a["dim"], 1.5, 0.4)
+        q, W, bs = p + ".right", r["width"], r["width"] // r["blocks"]
+        out[q + ".y"], out[q + ".x"], out[q + ".o"] = mat(W, width), mat(W, width), mat(width, W)
+        out[q + ".y.b"], out[q + ".x.b"] = vec(W, 0.0, 0.3), vec(W, 0.0, 0.3)
+        out[q + ".conv"], out[q + ".conv.b"] = 0.6 * torch.randn(W, r["conv"], generator=g, dtype=F64), vec(W, 0.0, 0.2)
+        for t in ("ra", "ri"):
+            out[f"{q}.{t}"] = torch.randn(r["blocks"], bs, bs, generator=g, dtype=F64) / math.sqrt(bs)
+            out[f"{q}.{t}.b"] = 0.5 * torch.randn(r["blocks"], bs, generator=g, dtype=F64)
+        out[q + ".lam"] = -3.0 + 2.0 * torch.randn(W, generator=g, dtype=F64)
+    elif layer["type"] == "latent_attention":
+        H, d, dr, dv = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
+        out[p + ".dq"], out[p + ".uq"] = mat(m["q_rank"], width), mat(H * (d + dr), m["q_rank"])
+        out[p + ".dkv"] = mat(m["kv_rank"] + dr, width)
+        out[p + ".uk"], out[p + ".uv"] = mat(H * d, m["kv_rank"]), mat(H * dv, m["kv_rank"])
+        out[p + ".g"], out[p + ".o"] = mat(H * dv, width), mat(width, H * dv)
+        out[p + ".dq.norm"], out[p + ".dkv.norm"] = vec(m["q_rank"]), vec(m["kv_rank"])
+    else:
+        H, G, d, dv, taps = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
+        out[p + ".q"], out[p + ".k"], out[p + ".v"] = mat(G * d, width), mat(G * d, width), mat(H * dv, width)
+        for t, n in (("q", G * d), ("k", G * d), ("v", H * dv)):
+            out[f"{p}.{t}.conv"] = 0.6 * torch.randn(n, taps, generator=g, dtype=F64)
+        out[p + ".b"], out[p + ".a"] = mat(H, width), mat(H, width)
+        out[p + ".A_log"], out[p + ".dt_bias"] = vec(H, -1.0, 1.0), vec(H, 0.0, 1.0)
+        out[p + ".norm"] = vec(dv)
+        out[p + ".g"], out[p + ".o"] = mat(H * dv, width), mat(width, H * dv)
+    if layer.get("mlp") is not None:
+        f = layer["mlp"]["ff"]
+        out[f"l{i}.norm2"] = vec(width)
+        out[f"l{i}.mlp.up"], out[f"l{i}.mlp.down"] = mat(f, width), mat(width, f)
+    return out
+
+
+def random_weights(cfg, seed):
+    """Weights of a size that keeps every mechanism in play: products of unit scale, decays
+    spread between forgetting at once and hardly at all."""
+    g = torch.Generator().manual_seed(seed)
+    width = cfg["width"]
+    w = {"embed": torch.randn(cfg["vocab"], width, generator=g, dtype=F64) / math.sqrt(width) * 2.0,
+         "final.norm": 1.0 + 0.2 * torch.randn(width, generator=g, dtype=F64)}
+    for i, layer in enumerate(cfg["layers"]):
+        if layer.get("weights_of") is None:
+            w.update(_layer_tensors(layer, i, width, g))
+    return w
