@@ -19,6 +19,7 @@ D1, P1, L1: one mixer each, alone, without feed-forward.
 """
 
 import json
+import math
 import os
 
 import torch
@@ -127,3 +128,80 @@ def read_weights(model_dir, as_stored_in=None):
 def tokens(cfg, n, seed):
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, cfg["vocab"], (n,), generator=g).tolist()
+
+
+# Sizes nearer to a real model's layers (N6, N7): heads of 64 and 128 on the matrix cores' kernels,
+# cached latent rows of several hundred elements, delta heads of 64 and 128.
+CONFIGS["N6"] = _cfg(200, 192, 1e-6, 1.5, [
+    delta(6, 3, 64, 96, 4, ff=128),
+    parallel(attn(6, 2, 64, rot=32, base=20000.0, scaling=(8.0, 1.0, 4.0, 64), window=48, keep=4), 256, 8, 4, ff=160),
+    latent(6, 64, 32, 64, 96, 160, base=3000.0, ff=128),
+    parallel(attn(6, 2, 64, rot=32, base=20000.0, scaling=(8.0, 1.0, 4.0, 64), window=48, keep=4), 256, 8, 4, ff=160,
+             weights_of=1)])
+CONFIGS["N7"] = _cfg(160, 128, 1e-5, 0.5, [
+    latent(3, 128, 64, 128, 72, 448, ff=96),
+    delta(2, 1, 128, 128, 4),
+    parallel(attn(4, 4, 128, vdim=128, rot=128, window=32, keep=1), 128, 2, 2, left_scale=0.5, right_scale=2.0)])
+# The same layer three times, the first of them running with the last one's tensors.
+CONFIGS["N8"] = _cfg(64, 48, 1e-5, 1.0, [
+    delta(2, 2, 16, 16, 2, ff=32, weights_of=2),
+    delta(2, 2, 16, 16, 2, ff=32, weights_of=2),
+    delta(2, 2, 16, 16, 2, ff=32)])
+
+
+def aimed_attention(cfg, w, query_token, key_token, strength=30.0):
+    """Changes ``w`` (weights of a model whose FIRST layer has windowed attention) so that, in
+    layer 0, the query of ``query_token`` looks along the key of ``key_token`` wherever it stands:
+    the two tokens get an embedding direction of their own each, which the query and key matrices
+    turn into one and the same long vector in the part of every head that does not rotate.  The
+    norm makes every query and key as long as any other, so the aimed score is about
+    sqrt(dim) times a random one; the value of ``key_token`` is unlike any other."""
+    m = cfg["layers"][0]["mixer"]["left"]
+    H, G, d = m["heads"], m["kv_heads"], m["dim"]
+    rot = (m.get("rot") or {}).get("dims", 0)
+    assert rot < d, "only the part of a head that does not rotate can be aimed"
+    width = cfg["width"]
+    g = torch.Generator().manual_seed(99)
+    a, b = torch.zeros(width, dtype=torch.float64), torch.zeros(width, dtype=torch.float64)
+    a[0], b[1] = 1.0, 1.0
+    w["embed"][:, :2] = 0.0
+    w["embed"][query_token, 0] = 1.0
+    w["embed"][key_token, 1] = 1.0
+    u = torch.randn(d - rot, generator=g, dtype=torch.float64)
+    p = "l0.mix.left"
+    for h in range(H):
+        w[p + ".q"][h * d + rot:(h + 1) * d] += strength * torch.outer(u, a)
+    for h in range(G):
+        w[p + ".k"][h * d + rot:(h + 1) * d] += strength * torch.outer(u, b)
+    w[p + ".v"] += 3.0 * torch.outer(torch.randn(w[p + ".v"].shape[0], generator=g, dtype=torch.float64), b)
+    return w
+
+
+def aimed_latent(cfg, w, query_token, key_token, strength=30.0, score=25.0):
+    """The same for a model whose FIRST layer is latent attention: channel 0 of both latents is
+    the aimed tokens' own, and the up-projections turn it into one vector in the unrotated
+    part of every head, of a length that makes the aimed score ``score``."""
+    m = cfg["layers"][0]["mixer"]
+    H, d, dr, rank, q_rank = m["heads"], m["dim"], m["rot_dim"], m["kv_rank"], m["q_rank"]
+    g = torch.Generator().manual_seed(98)
+    w["embed"][:, :2] = 0.0
+    w["embed"][query_token, 0] = 1.0
+    w["embed"][key_token, 1] = 1.0
+    p = "l0.mix"
+    w[p + ".dq"][0] = 0.0
+    w[p + ".dq"][0, 0] = strength
+    w[p + ".dkv"][0] = 0.0
+    w[p + ".dkv"][0, 1] = strength
+    w[p + ".dq"][1:, 0] = 0.0
+    w[p + ".dkv"][1:, 1] = 0.0
+    u = torch.randn(d, generator=g, dtype=torch.float64)
+    u = u / u.norm()
+    # after the norms channel 0 holds about sqrt(q_rank) g_q[0] and sqrt(rank) g_c[0]
+    amp = math.sqrt(score / (float(m["scale"]) * math.sqrt(q_rank * rank)
+                             * abs(float(w[p + ".dq.norm"][0] * w[p + ".dkv.norm"][0]))))
+    for h in range(H):
+        w[p + ".uq"][h * (d + dr):h * (d + dr) + d, 0] = amp * u
+        w[p + ".uq"][h * (d + dr) + d:(h + 1) * (d + dr), 0] = 0.0
+        w[p + ".uk"][h * d:(h + 1) * d, 0] = amp * u
+    w[p + ".uv"][:, 0] = 2.0 * torch.randn(w[p + ".uv"].shape[0], generator=g, dtype=torch.float64)
+    return w
