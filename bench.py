@@ -20,6 +20,9 @@ Other workloads, each printing one JSON line of its own (``--model`` chooses the
                                prefilled in portions of --chunk tokens beside decode tokens
     --workload ribovik         prefill and decode of a Ribovik model (chunked attention with a sink, a dense
                                layer and layers of routed experts) beside a Llama model of the same sizes
+    --workload natenex         prefill and decode of a Natenex model (windowed attention that keeps the first
+                               positions beside a gated linear recurrence, a gated delta rule, attention through
+                               latents) beside a Nusilix and a Llama model of the same layer sizes
     --workload nusilix         prefill and decode of a Nusilix model (every fourth layer recurrent)
                                beside a Llama model of the same layer sizes (--sizes NAME; all if
                                not given)
@@ -55,8 +58,8 @@ def main(argv=None):
     ap.add_argument("--model", default="tinyllama-1.1b", choices=["tinyllama-1.1b", "llama2-7b", "llama3-8b"],
                     help="whose sizes to run (the default is the headline configuration)")
     ap.add_argument("--extra", default="", help="engine options for experiments: key=value,key=value (ints or words)")
-    ap.add_argument("--workload", default="headline", choices=["headline", "decode-run", "prefill-chunks", "mixed", "nusilix", "ribovik"])
-    ap.add_argument("--sizes", default="", help="layer sizes of the nusilix and ribovik workloads (see benchmark.NUSILIX_SIZES)")
+    ap.add_argument("--workload", default="headline", choices=["headline", "decode-run", "prefill-chunks", "mixed", "nusilix", "ribovik", "natenex"])
+    ap.add_argument("--sizes", default="", help="layer sizes of the nusilix, ribovik and natenex workloads (see benchmark.NUSILIX_SIZES)")
     ap.add_argument("--chunk", type=int, default=512, help="tokens per prompt portion (prefill-chunks, mixed)")
     ap.add_argument("--requests", type=int, default=32, help="requests of the mixed workload")
     ap.add_argument("--new-tokens", type=int, default=64, help="tokens each request of the mixed workload generates")
@@ -91,7 +94,7 @@ def main(argv=None):
     for item in filter(None, args.extra.split(",")):
         key, _, val = item.partition("=")
         extra[key] = int(val) if val.lstrip("-").isdigit() else (val or True)
-    if args.workload in ("nusilix", "ribovik"):
+    if args.workload in ("nusilix", "ribovik", "natenex"):
         names = [args.sizes] if args.sizes else sorted(B.NUSILIX_SIZES)
         res = {"workload": args.workload, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
                "weights": "random", "context": args.context}

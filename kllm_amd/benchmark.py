@@ -362,6 +362,30 @@ def ribovik_config(width, heads, kv_heads, head_dim, ff, layers, vocab, experts=
     return {"architecture": "Ribovik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "layers": entries}
 
 
+# Natenex beside Nusilix and Llama: the attention half of its 'parallel' layers has Llama's sizes
+# behind a window of half the context that keeps the first four positions, beside a recurrence as
+# wide as the model in blocks of 256; its delta layers have width / 128 heads with keys and values
+# of 128 on half as many key heads; its latent layers cache rows of 512 + 64 for heads of
+# 128 + 64 with values of 128.  The layers come in fours: parallel, parallel, delta, latent.
+def natenex_config(width, heads, kv_heads, head_dim, ff, layers, vocab, window=1024, keep_first=4) -> dict:
+    mlp = {"kind": "dense", "ff": ff}
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+            "mask": {"size": window, "keep_first": keep_first},
+            "rot": {"base": 500000.0, "dims": head_dim // 2,
+                    "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 1024}}}
+    parallel = {"type": "parallel", "mlp": mlp,
+                "mixer": {"left": left, "right": {"width": width, "blocks": max(1, width // 256), "conv": 4},
+                          "left_scale": 1.0, "right_scale": 1.0}}
+    delta = {"type": "delta", "mlp": mlp,
+             "mixer": {"heads": width // 128, "kv_heads": max(1, width // 256), "dim": 128, "vdim": 128, "conv": 4}}
+    latent = {"type": "latent_attention", "mlp": mlp,
+              "mixer": {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "q_rank": 3 * width // 4, "kv_rank": 512,
+                        "scale": 192 ** -0.5, "rot": {"base": 10000.0, "dims": 64}}}
+    cycle = (parallel, parallel, delta, latent)
+    return {"architecture": "Natenex", "vocab": vocab, "width": width, "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-6}, "layers": [dict(cycle[i % 4]) for i in range(layers)]}
+
+
 def spread_routing(eng: Engine, seed: int = 0) -> None:
     """Random weights as the engine draws them (all small, corrections all near 1) send every
     token to the same experts.  A router with large weights and no correction spreads the
@@ -382,15 +406,20 @@ def spread_routing(eng: Engine, seed: int = 0) -> None:
 
 def measure_design_pair(sizes: dict, dtype: str, batches=(1, 8), context: int = 2048, prompt: int = 2048,
                         steps: int = 64, delta_every: int = 4, design: str = "nusilix", design_sizes=None) -> dict:
-    """Prefill and decode throughput of a model of ``design`` ("nusilix", "ribovik") and of a
-    Llama model of the same layer sizes, one after the other on this GPU."""
+    """Prefill and decode throughput of a model of ``design`` ("nusilix", "ribovik", "natenex") and
+    of a Llama model of the same layer sizes (for Natenex a Nusilix model too, the nearest in
+    kind), one after the other on this GPU."""
     import gc
     out = {}
+    models = []
     if design == "ribovik":
         first = ribovik_config(**sizes, **(design_sizes or {}), chunk=max(4096, context + 64))
+    elif design == "natenex":
+        first = natenex_config(**sizes, window=max(64, context // 2))
+        models.append(("nusilix", nusilix_config(delta_every=delta_every, **sizes)))
     else:
         first = nusilix_config(delta_every=delta_every, **sizes)
-    for name, cfg in ((design, first), ("llama", llama_config(**sizes))):
+    for name, cfg in [(design, first)] + models + [("llama", llama_config(**sizes))]:
         eng = make_engine(cfg, dtype, max_tokens=max(batches) * context + 2 * prompt, max_model_len=context + 64,
                           max_requests=max(batches))
         spread_routing(eng)

@@ -59,7 +59,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ span_of_token,
     const int* __restrict__ block_table, int max_pages, int page_size, int H, int KV, int window, int chunk, int sink,
-    float scale, const float* __restrict__ slopes, int head_tiles, const int* __restrict__ token_list) {
+    int keep_first, float scale, const float* __restrict__ slopes, int head_tiles, const int* __restrict__ token_list) {
   constexpr int hd = 16 * HDT;
   constexpr int KS = (hd + 31) / 32;           // MFMA steps over head_dim for the scores
   constexpr int kDecodeAhead = decode_ahead(HDT);
@@ -74,7 +74,11 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
   const int len = positions[t] + 1;
   const int start = first_key(len - 1, window, chunk);     // window and chunked mask
   const int first = start / 32 * 32;                       // tiles of 32 keys from here
-  const int tiles = (len - first + 31) / 32;
+  // Kept first positions: the keys below kept_end (none of them in the window's tiles) come
+  // first, in n_kept tiles of their own from key 0; pages between them and the window may be gone.
+  const int kept_end = min(keep_first, first);
+  const int n_kept = (kept_end + 31) / 32;
+  const int tiles = (len - first + 31) / 32 + n_kept;
   const int per = (tiles + nslices - 1) / nslices;
   const int tile0 = slice * per, tile1 = min(tile0 + per, tiles);
   const int* table = block_table + (long)span_of_token[t] * max_pages;
@@ -112,9 +116,14 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
   // Loads carry no branch: a tile or a page that does not exist reads a valid address
   // (table entry 0, page 0) and is marked dead, so that the compiler can count the loads in
   // flight and a tile's arithmetic waits for its own operands only.
+  auto tile_key = [&](int tile) { return tile < n_kept ? tile * 32 : first + (tile - n_kept) * 32; };
+  // a key of tile `tile` is read: below kept_end in a kept tile; in the window, or kept, in the others
+  auto key_read = [&](int tile, int key) {
+    return tile < n_kept ? key < kept_end : (key < len && (key >= start || key < keep_first));
+  };
   auto page_of = [&](int tile, int u) -> int {
-    const int k0 = first + tile * 32 + 16 * u;
-    const bool ok = tile < tile1 && k0 < len && k0 + 16 > start;
+    const int k0 = tile_key(tile) + 16 * u;
+    const bool ok = tile < tile1 && (tile < n_kept ? k0 < kept_end : (k0 < len && (k0 + 16 > start || k0 < keep_first)));
     const int page = table[ok ? k0 / page_size : 0];
     return ok ? page : -1;
   };
@@ -123,7 +132,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int page = u ? page1 : page0;
-      const int k0 = first + tile * 32 + 16 * u;
+      const int k0 = tile_key(tile) + 16 * u;
       T.live[u] = page >= 0;
       const long base = ((long)(T.live[u] ? page : 0) * 2 * KV + kvh) * block;
       const bf16_t* kp = cache + base + (long)(k0 % page_size + c) * hd;        // keys [slot][hd]
@@ -156,8 +165,8 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
     pg[j][1] = page_of(tile0 + kDecodeAhead + j, 1);
   }
   auto compute = [&](const Tile& cur, int tile) {
-    const int kb = first + tile * 32;
-    const bool edge = kb < start || kb + 32 > len;
+    const int kb = tile_key(tile);
+    const bool edge = tile < n_kept || kb < start || kb + 32 > len;
     floatx4 s[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
@@ -175,7 +184,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int key = kb + 16 * u + 4 * g + i;
-        const bool ok = cur.live[u] && key >= start && key < len;
+        const bool ok = cur.live[u] && key_read(tile, key);
         float sc = s[u][i] * scale;
         if (BIASED) sc -= slope * (float)(len - 1 - key);      // (a constant of the code: a model without slopes has none of it)
         s[u][i] = ok ? sc : -INFINITY;
@@ -207,7 +216,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = kb + 16 * u + 4 * g + i;
-          const bool ok = cur.live[u] && (!edge || (key >= start && key < len));   // stale slots may hold anything
+          const bool ok = cur.live[u] && (!edge || key_read(tile, key));   // stale slots may hold anything
           a[4 * u + i] = ok ? cur.v[u][r][i] : (bf16_t)0.f;
         }
       acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[r], 0, 0, 0);
@@ -287,7 +296,7 @@ template <int HDT, int W>
 static int launch_decode(dim3 grid, hipStream_t stream, const void* q, void* out, float* part,
                          const void* cache, const int* positions, const int* span_of_token,
                          const int* block_table, int max_pages, int page_size, int H, int KV, int window, int chunk, int sink,
-                         float scale, const float* slopes, int head_tiles, const int* token_list) {
+                         int keep_first, float scale, const float* slopes, int head_tiles, const int* token_list) {
   const int heads = H / KV < 16 ? H / KV : 16;
   const size_t lds = (size_t)W * heads * (16 * HDT + 4) * sizeof(float);
   static int raised = 0;
@@ -309,12 +318,12 @@ static int launch_decode(dim3 grid, hipStream_t stream, const void* q, void* out
     }
     hipLaunchKernelGGL((attn_decode_mfma_kernel<HDT, W, true>), grid, dim3(64 * W), lds, stream,
                        (const bf16_t*)q, (bf16_t*)out, part, (const bf16_t*)cache, positions, span_of_token,
-                       block_table, max_pages, page_size, H, KV, window, chunk, sink, scale, slopes, head_tiles, token_list);
+                       block_table, max_pages, page_size, H, KV, window, chunk, sink, keep_first, scale, slopes, head_tiles, token_list);
     return 0;
   }
   hipLaunchKernelGGL((attn_decode_mfma_kernel<HDT, W>), grid, dim3(64 * W), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, part, (const bf16_t*)cache, positions, span_of_token,
-                     block_table, max_pages, page_size, H, KV, window, chunk, sink, scale, slopes, head_tiles, token_list);
+                     block_table, max_pages, page_size, H, KV, window, chunk, sink, keep_first, scale, slopes, head_tiles, token_list);
   return 0;
 }
 
@@ -411,13 +420,15 @@ extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, 
 static int attn_decode_run(const char* who, const void* q, void* out, float* part, long part_floats,
                            const void* cache, const int* positions, const int* span_of_token,
                            const int* block_table, int max_pages, int page_size, int n, int H, int KV,
-                           int hd, int window, int chunk, int sink, float scale, const float* slopes, int nslices, int dtype,
+                           int hd, int window, int chunk, int sink, int keep_first, float scale, const float* slopes, int nslices, int dtype,
                            const int* token_list, int n_listed, hipStream_t stream) {
   KLLM_REQUIRE(q && out && part && cache && positions && span_of_token && block_table,
                "%s: null pointer", who);
   KLLM_REQUIRE(dtype == DT_BF16 || dtype == DT_F32, "%s: unknown dtype %d", who, dtype);
   KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && H % KV == 0, "%s: bad heads n=%d H=%d KV=%d", who, n, H, KV);
+  KLLM_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "%s: kept first positions (%d) go with a window", who, keep_first);
   if (dtype == DT_F32) {
+    KLLM_REQUIRE(keep_first == 0, "%s: the 32-bit kernels read one run of keys a query", who);
     KLLM_REQUIRE(max_pages > 0 && window >= 0 && chunk >= 0, "%s: bad table width, window or chunk", who);
     KLLM_REQUIRE(nslices >= 1 && part_floats >= (long)n * H * nslices * (hd + 2),
                  "%s: the partial results of n=%d H=%d nslices=%d head_dim=%d need %ld floats, the workspace has %ld",
@@ -450,11 +461,11 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
     if (int rc = nslices == 1                                                                     \
                      ? launch_decode<HDT, decode_waves_whole(HDT)>(                               \
                            grid, stream, q, out, part, cache, positions, span_of_token,           \
-                           block_table, max_pages, page_size, H, KV, window, chunk, sink, scale, slopes,          \
+                           block_table, max_pages, page_size, H, KV, window, chunk, sink, keep_first, scale, slopes,          \
                            head_tiles, token_list)                                                            \
                      : launch_decode<HDT, kDecodeWavesShared>(                                    \
                            grid, stream, q, out, part, cache, positions, span_of_token,           \
-                           block_table, max_pages, page_size, H, KV, window, chunk, sink, scale, slopes,          \
+                           block_table, max_pages, page_size, H, KV, window, chunk, sink, keep_first, scale, slopes,          \
                            head_tiles, token_list))                                                           \
       return rc;                                                                                  \
     break
@@ -474,10 +485,10 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
 extern "C" int kllm_attn_decode(const void* q, void* out, float* part, long part_floats,
                                 const void* cache, const int* positions, const int* span_of_token,
                                 const int* block_table, int max_pages, int page_size, int n, int H,
-                                int KV, int hd, int window, int chunk, int sink, float scale, const float* slopes, int nslices, int dtype,
+                                int KV, int hd, int window, int chunk, int sink, int keep_first, float scale, const float* slopes, int nslices, int dtype,
                                 const int* token_list, int n_listed, hipStream_t stream) {
   return attn_decode_run("attn_decode", q, out, part, part_floats, cache, positions, span_of_token,
-                         block_table, max_pages, page_size, n, H, KV, hd, window, chunk, sink, scale, slopes, nslices, dtype,
+                         block_table, max_pages, page_size, n, H, KV, hd, window, chunk, sink, keep_first, scale, slopes, nslices, dtype,
                          token_list, n_listed, stream);
 }
 
@@ -544,6 +555,6 @@ extern "C" int kllm_attn_decode_static(const void* q, void* out, const void* cac
   // Nothing in the scratch has to start at zero: the first kernel writes every partial result
   // (maximum, sum, output of each token, head and slice) that the second one reads.
   return attn_decode_run("attn_decode_static", q, out, part, (long)KLLM_ATTN_DECODE_STATIC_FLOATS, cache,
-                         positions, span_of_token, block_table, max_pages, page_size, n, H, KV, hd, window, 0, 0,
+                         positions, span_of_token, block_table, max_pages, page_size, n, H, KV, hd, window, 0, 0, 0,
                          scale, nullptr, nslices, dtype, token_list, n_listed, stream);
 }

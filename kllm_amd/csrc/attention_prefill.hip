@@ -75,7 +75,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ query_tiles, int n_tiles, const int* __restrict__ span_start,
     const int* __restrict__ span_pos, const int* __restrict__ block_table, int max_pages,
-    int page_size, unsigned page_magic, int H, int KV, int window, int chunk, int sink, float scale, const float* __restrict__ slopes, float* __restrict__ part) {
+    int page_size, unsigned page_magic, int H, int KV, int window, int chunk, int sink, int keep_first, float scale, const float* __restrict__ slopes, float* __restrict__ part) {
   typedef PrefillShape<HDT> S;
   constexpr int hd = S::hd, KS = S::KS, NB = S::NB, KT = S::KT, KLD = S::KLD, VLD = S::VLD, CPT = S::CPT;
   extern __shared__ __attribute__((aligned(16))) bf16_t tiles_lds[];   // [PAR][2][kBuf]
@@ -134,13 +134,20 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     for (int i = 0; i < 16; ++i) acc[r][i] = 0.f;
 
   const int kb0 = lowest / 32 * 32;
-  const int ntiles_all = (blk_qmax - kb0) / KT + 1;
+  // Kept first positions: the keys below kept_end (none of them in the tiles from kb0 on) come
+  // first, in n_kept tiles of their own from key 0; pages between them and kb0 may be gone.
+  const int kept_end = min(keep_first, kb0);
+  const int n_kept = (kept_end + KT - 1) / KT;
+  const int ntiles_all = (blk_qmax - kb0) / KT + 1 + n_kept;
   // The tiles go in turn to the slices (workgroups of the same block and head, blockIdx.y: where
   // the blocks alone leave CUs idle) and, within a slice, to the groups of waves.
   const int nslices = gridDim.y, slice = blockIdx.y;
   const int ntiles = (ntiles_all + PAR * nslices - 1) / (PAR * nslices);   // steps of the loop: the same for all
   auto tile_no = [&](int t) { return nslices * (PAR * t + par) + slice; };
-  auto tile_key = [&](int t) { return kb0 + KT * tile_no(t); };   // first key of this group's t-th tile
+  auto tile_key = [&](int t) {                                    // first key of this group's t-th tile
+    const int n = tile_no(t);
+    return n < n_kept ? KT * n : kb0 + KT * (n - n_kept);
+  };
   // page and slot of a key: a shift and a mask when the page size is a power of two
   // Page of a key without a division: page_magic = ceil(2^35 / page_size) from the host, exact
   // for keys below 2^24 and pages of up to 2,048 tokens (kPrefillMaxKeys, checked at the launch).
@@ -173,7 +180,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
   struct Stage {
     bf16x8 k[CPT], v[CPT];
   };
-  auto key_ok = [&](int key) { return key < kv_len && key >= first_page_key; };
+  auto key_ok = [&](int key) { return key < kv_len && (key >= first_page_key || key < keep_first); };   // (kept positions' pages stay)
   auto lookup = [&](int t) -> Pages {
     Pages P;
 #pragma unroll
@@ -258,7 +265,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     l = 1.f;
     m_limit = grow_raw;
   }
-  auto tile_math = [&](auto masked, int kb, const bf16_t* buf) {
+  auto tile_math = [&](auto masked, int kb, const bf16_t* buf, bool kept_tile) {
     // ---- scores: this lane's key rows are kb + c and kb + 32 + c
     floatx16 s[NB];
 #pragma unroll
@@ -276,13 +283,17 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
         for (int i = 0; i < 16; ++i) s[b][i] += fmaf(sb, (float)(32 * b + 8 * (i / 4) + i % 4), base);
     }
     if constexpr (decltype(masked)::value) {
-      const int hi = min(qpos, kv_len - 1) - kb - 4 * g, lo = my_start - kb - 4 * g;   // offsets in the tile this lane's query reads
+      // offsets in the tile this lane's query reads: up to hi, and from lo on or below kf (a kept
+      // tile: below kept_end only, the rest of it is the window's tiles' or masked)
+      const int hi = min(qpos, kv_len - 1) - kb - 4 * g;
+      const int lo = kept_tile ? KT : my_start - kb - 4 * g;
+      const int kf = (kept_tile ? kept_end : keep_first) - kb - 4 * g;
 #pragma unroll
       for (int b = 0; b < NB; ++b)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int e = 32 * b + 8 * (i / 4) + i % 4;
-          const bool ok = (e <= hi) & (e >= lo);
+          const bool ok = (e <= hi) & ((e >= lo) | (e < kf));
           s[b][i] = ok ? s[b][i] : -INFINITY;
         }
     }
@@ -357,11 +368,13 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
   const int w_highstart = first_key(w_qmax, window, chunk);   // from here on no query of the wave masks a key below it
   auto compute = [&](int t, const bf16_t* buf) {
     const int kb = tile_key(t);
-    if (!active || kb > w_qmax || kb + KT <= w_lowest) return;   // nothing here for this wave's queries
-    if (HDT <= 4 && kb >= w_highstart && kb + KT - 1 <= w_qmin)   // every key for every query of the wave
-      tile_math(std::false_type(), kb, buf);
+    const bool kept_tile = tile_no(t) < n_kept;                  // kept positions: for every query behind them
+    // nothing here for this wave's queries: beyond their last, or below their first and without a kept position
+    if (!active || (!kept_tile && (kb > w_qmax || (kb + KT <= w_lowest && kb >= keep_first)))) return;
+    if (HDT <= 4 && !kept_tile && kb >= w_highstart && kb + KT - 1 <= w_qmin)   // every key for every query of the wave
+      tile_math(std::false_type(), kb, buf, false);
     else
-      tile_math(std::true_type(), kb, buf);
+      tile_math(std::true_type(), kb, buf, kept_tile);
   };
 
   // Tiles in registers on their way to LDS: two for head size 96; one for the small heads, whose
@@ -755,7 +768,7 @@ template <int HDT, int PAR>
 static void launch_prefill_par(int grid, hipStream_t stream, const void* q, void* out, const void* cache,
                                const int* query_tiles, int n_tiles, const int* span_start,
                                const int* span_pos, const int* block_table, int max_pages, int page_size,
-                               int H, int KV, int window, int chunk, int sink, float scale, const float* slopes, float* part = nullptr, int nslices = 1) {
+                               int H, int KV, int window, int chunk, int sink, int keep_first, float scale, const float* slopes, float* part = nullptr, int nslices = 1) {
   typedef PrefillShape<HDT> S;
   const size_t lds = (size_t)PAR * 2 * S::kBuf * sizeof(bf16_t);   // also holds the groups' merge
   static int raised = 0;
@@ -767,7 +780,7 @@ static void launch_prefill_par(int grid, hipStream_t stream, const void* q, void
   const unsigned page_magic = (unsigned)(((1UL << 35) + page_size - 1) / page_size);   // ceil(2^35 / page_size)
   hipLaunchKernelGGL((attn_prefill_mfma_kernel<HDT, PAR>), dim3(grid, nslices), dim3(64 * kPrefillWaves * PAR), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, query_tiles, n_tiles,
-                     span_start, span_pos, block_table, max_pages, page_size, page_magic, H, KV, window, chunk, sink, scale, slopes, part);
+                     span_start, span_pos, block_table, max_pages, page_size, page_magic, H, KV, window, chunk, sink, keep_first, scale, slopes, part);
   if (nslices > 1) {
     const dim3 mgrid(n_tiles * kQueryBlock, ceil_div(H, kMergeWaves));
     hipLaunchKernelGGL((attn_prefill_merge_kernel<(HDT + 1) / 2>), mgrid, dim3(64 * kMergeWaves), 0, stream,
@@ -814,7 +827,7 @@ template <int HDT>
 static void launch_prefill(int grid, hipStream_t stream, const void* q, void* out, const void* cache,
                            const int* query_tiles, int n_tiles, const int* span_start,
                            const int* span_pos, const int* block_table, int max_pages, int page_size,
-                           int H, int KV, int window, int chunk, int sink, float scale, const float* slopes, long keys_total,
+                           int H, int KV, int window, int chunk, int sink, int keep_first, float scale, const float* slopes, long keys_total,
                            int keys_longest, float* part, int nslices) {
   const int cus = device_cus();
   // (the caller asked kllm_attn_prefill_slices: few blocks of a large head.  The slices' results
@@ -823,7 +836,7 @@ static void launch_prefill(int grid, hipStream_t stream, const void* q, void* ou
   if (nslices > 1 && keys_longest >= kPrefillSliceFromKeys) {
     launch_prefill_par<HDT, PrefillShape<HDT>::kMaxPar>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start,
                                                         span_pos, block_table, max_pages, page_size, H, KV, window, chunk, sink,
-                                                        scale, slopes, part, nslices);
+                                                        keep_first, scale, slopes, part, nslices);
     return;
   }
   bool chain_bound = true;
@@ -831,11 +844,11 @@ static void launch_prefill(int grid, hipStream_t stream, const void* q, void* ou
     chain_bound = 5 * (keys_total * H / cus) < 6 * (long)keys_longest;
   if (grid > 2 * cus || PrefillShape<HDT>::kMaxPar == 1 || (grid > cus && !chain_bound))
     launch_prefill_par<HDT, 1>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,
-                               block_table, max_pages, page_size, H, KV, window, chunk, sink, scale, slopes);
-  else if (HDT >= 4 || 4 * grid > 3 * cus)
+                               block_table, max_pages, page_size, H, KV, window, chunk, sink, keep_first, scale, slopes);
+  else if (HDT >= 4 || 4 * grid > 3 * cus || keep_first > 0)   // (the kernel below reads one run of keys a query)
     launch_prefill_par<HDT, PrefillShape<HDT>::kMaxPar>(grid, stream, q, out, cache, query_tiles, n_tiles,
                                                         span_start, span_pos, block_table, max_pages, page_size,
-                                                        H, KV, window, chunk, sink, scale, slopes);
+                                                        H, KV, window, chunk, sink, keep_first, scale, slopes);
   else
     launch_prefill_split<HDT>(n_tiles, stream, q, out, cache, query_tiles, span_start, span_pos, block_table,
                               max_pages, page_size, H, KV, window, chunk, sink, scale, slopes);
@@ -864,7 +877,7 @@ extern "C" int kllm_attn_prefill_slices(int n_tiles, int H, int hd) {
 extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,
                                  int n_tiles, const int* span_start, const int* span_pos,
                                  const int* block_table, int max_pages, int page_size, int H, int KV,
-                                 int hd, int window, int chunk, int sink, float scale, const float* slopes, long keys_total, int keys_longest,
+                                 int hd, int window, int chunk, int sink, int keep_first, float scale, const float* slopes, long keys_total, int keys_longest,
                                  float* part, long part_floats, int nslices, int n_rows, int dtype, hipStream_t stream) {
   KLLM_REQUIRE(q && out && cache && query_tiles && span_start && span_pos && block_table,
                "attn_prefill: null pointer");
@@ -872,7 +885,9 @@ extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, co
   KLLM_REQUIRE(dtype == DT_BF16 || dtype == DT_F32, "attn_prefill: unknown dtype %d", dtype);
   KLLM_REQUIRE(n_tiles > 0 && H > 0 && KV > 0 && H % KV == 0, "attn_prefill: bad sizes tiles=%d H=%d KV=%d",
                n_tiles, H, KV);
+  KLLM_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "attn_prefill: kept first positions (%d) go with a window", keep_first);
   if (dtype == DT_F32) {
+    KLLM_REQUIRE(keep_first == 0, "attn_prefill: the 32-bit kernels read one run of keys a query");
     KLLM_REQUIRE(max_pages > 0 && window >= 0 && chunk >= 0, "attn_prefill: bad table width, window or chunk");
     return attn_f32_prefill((const float*)q, (float*)out, (const float*)cache, query_tiles, n_tiles, span_start,
                             span_pos, block_table, max_pages, page_size, H, KV, hd, window, chunk, sink, scale, slopes, stream);
@@ -897,7 +912,7 @@ extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, co
 #define KLLM_PF(HDT)                                                                              \
   case HDT:                                                                                       \
     launch_prefill<HDT>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,  \
-                        block_table, max_pages, page_size, H, KV, window, chunk, sink, scale, slopes, keys_total, \
+                        block_table, max_pages, page_size, H, KV, window, chunk, sink, keep_first, scale, slopes, keys_total, \
                         keys_longest, part, nslices);                                             \
     break
   switch (hd / 32) {

@@ -233,11 +233,12 @@ int kllm_attn_generic(const void* q, void* out, const void* cache, const int* po
 int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, int max_keys);
 /* Whether the float32 attention on the matrix cores takes this head size and page size. */
 int kllm_attn_f32_fits(int hd, int page_size);
-/* `chunk` and `sink` in kllm_attn_decode and kllm_attn_prefill: as in kllm_attn_generic. */
+/* `chunk`, `sink` and `keep_first` in kllm_attn_decode and kllm_attn_prefill: as in kllm_attn_generic
+ * (kept first positions: bfloat16 only). */
 int kllm_attn_decode(const void* q, void* out, float* part, long part_floats, const void* cache,
                      const int* positions, const int* span_of_token, const int* block_table,
                      int max_pages, int page_size, int n, int H, int KV, int hd, int window,
-                     int chunk, int sink, float scale, const float* slopes, int nslices, int dtype,
+                     int chunk, int sink, int keep_first, float scale, const float* slopes, int nslices, int dtype,
                      const int* token_list, int n_listed, hipStream_t stream);
 
 /* kllm_attn_decode without a workspace argument and without any allocation: for callers
@@ -270,7 +271,7 @@ int kllm_attn_decode_static(const void* q, void* out, const void* cache, const i
 int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,
                       int n_tiles, const int* span_start, const int* span_pos,
                       const int* block_table, int max_pages, int page_size, int H, int KV, int hd,
-                      int window, int chunk, int sink, float scale, const float* slopes, long keys_total,
+                      int window, int chunk, int sink, int keep_first, float scale, const float* slopes, long keys_total,
                       int keys_longest, float* part, long part_floats, int nslices, int n_rows, int dtype,
                       hipStream_t stream);
 /* nslices of kllm_attn_prefill: how many workgroups share out the keys of a block and head

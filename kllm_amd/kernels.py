@@ -136,8 +136,8 @@ def _declare(lib):
         "kllm_calibrate_read": [P, L, P, P],
         "kllm_calibrate_read_workgroups": [],
         "kllm_calibrate_mfma": [I, I, P, P, P],
-        "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, I, I, P, I, P],
-        "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, P, L, I, P, L, I, I, I, P],
+        "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F, P, I, I, P, I, P],
+        "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, P, L, I, P, L, I, I, I, P],
         "kllm_attn_prefill_slices": [I, I, I],
         "kllm_gemm_act": [P, P, P, I, I, I, I, I, P, P],
         "kllm_add_sinusoid": [P, P, I, I, D, P],
@@ -184,7 +184,7 @@ LAUNCHING = ("kllm_embed", "kllm_add_rmsnorm", "kllm_rope_tables", "kllm_rope_ap
              "kllm_conv_state_update", "kllm_gated_delta_prep", "kllm_gated_delta_scan", "kllm_linear_recurrence_prep",
              "kllm_linear_recurrence_scan", "kllm_latent_kv_append", "kllm_latent_norm", "kllm_latent_query", "kllm_attn_latent",
              "kllm_latent_out", "kllm_scaled_sum")
-DYNAMIC_ARGS = {"kllm_attn_prefill": (18, 19)}     # arguments that may be a StepValue
+DYNAMIC_ARGS = {"kllm_attn_prefill": (19, 20)}     # arguments that may be a StepValue
 STRUCT_ARGS = {"kllm_gemv_plain": (7,), "kllm_gemv_swiglu": (8,), "kllm_gemv_rope_append": (17,),
                "kllm_fused_linear": (2,)}
 
@@ -1136,7 +1136,7 @@ def attn_prefill_slices(n_tiles, n_heads, head_dim, dtype=torch.bfloat16) -> int
 
 def attn_prefill(q, out, cache, query_tiles, n_tiles, span_start, span_pos, block_table, page_size,
                  n_heads, n_kv_heads, head_dim, window, scale, keys_total=0, keys_longest=0, part=None,
-                 nslices=None, slopes=None, chunk=0, sink=False):
+                 nslices=None, slopes=None, chunk=0, sink=False, keep_first=0):
     """query_tiles [n_tiles, 2] int32: (first token row, span) of each block of up to
     PREFILL_QUERY_BLOCK consecutive tokens of one span.  ``keys_total`` and
     ``keys_longest``: how many keys the blocks read, all together and the longest block
@@ -1163,7 +1163,7 @@ def attn_prefill(q, out, cache, query_tiles, n_tiles, span_start, span_pos, bloc
         _ptr(query_tiles, "attn query_tiles", torch.int32), n_tiles,
         _ptr(span_start, "attn span_start", torch.int32), _ptr(span_pos, "attn span_pos", torch.int32),
         _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size,
-        n_heads, n_kv_heads, head_dim, int(window), int(chunk), int(bool(sink)), float(scale),
+        n_heads, n_kv_heads, head_dim, int(window), int(chunk), int(bool(sink)), int(keep_first), float(scale),
         _slopes(slopes, n_heads, "attn_prefill"),
         keys_total if type(keys_total) is StepValue else int(keys_total),
         keys_longest if type(keys_longest) is StepValue else int(keys_longest),
@@ -1173,7 +1173,7 @@ def attn_prefill(q, out, cache, query_tiles, n_tiles, span_start, span_pos, bloc
 
 def attn_decode(q, out, part, cache, positions, span_of_token, block_table, page_size, n_heads,
                 n_kv_heads, head_dim, window, scale, nslices, token_list=None, n_listed=0, slopes=None, chunk=0,
-                sink=False):
+                sink=False, keep_first=0):
     n = q.shape[0]
     if (tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape)
             or q.dtype != cache.dtype or out.dtype != q.dtype):
@@ -1186,7 +1186,7 @@ def attn_decode(q, out, part, cache, positions, span_of_token, block_table, page
         part.numel(), _ptr(cache, "attn cache"), _ptr(positions, "attn positions", torch.int32),
         _ptr(span_of_token, "attn span_of_token", torch.int32),
         _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size, n,
-        n_heads, n_kv_heads, head_dim, int(window), int(chunk), int(bool(sink)), float(scale),
+        n_heads, n_kv_heads, head_dim, int(window), int(chunk), int(bool(sink)), int(keep_first), float(scale),
         _slopes(slopes, n_heads, "attn_decode"),
         int(nslices), dtype_code(q.dtype),
         _ptr(token_list, "attn token_list", torch.int32, True), int(n_listed), _stream())

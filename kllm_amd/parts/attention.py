@@ -231,9 +231,10 @@ class CausalSelfAttention(Part):
             prompt_ok = self.head_dim in K.PREFILL_HEAD_DIMS
         else:
             fast = prompt_ok = K.attn_f32_fits(self.head_dim, cache.page_size)
-        # the kernels on the matrix cores take keys and values of one width, and one run of keys a query
+        # the kernels on the matrix cores take keys and values of one width; the 32-bit ones one run of
+        # keys a query (no kept first positions)
         fast = (fast and mode != "generic" and self.value_dim == self.head_dim and not self.FAST_KERNELS_OFF
-                and not self.keep_first)
+                and not (self.keep_first and q.dtype != torch.bfloat16))
         if not fast:
             K.attn_generic(q, out, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
                            cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,
@@ -260,7 +261,8 @@ class CausalSelfAttention(Part):
             K.attn_prefill(q, out, cache.pages, blocks, n_blocks, ctx.span_start,
                            ctx.span_pos, cache.block_table, cache.page_size, self.heads,
                            self.kv_heads, self.head_dim, self.window, self.scale, total, longest, part=part,
-                           nslices=slices, slopes=self.slopes, chunk=self.chunk, sink=self.sink)
+                           nslices=slices, slopes=self.slopes, chunk=self.chunk, sink=self.sink,
+                           keep_first=self.keep_first)
 
     def _keys_read(self, ctx):
         """The step's key counts (see ``step_values``), as the engine worked them out for this
@@ -282,14 +284,15 @@ class CausalSelfAttention(Part):
             pages *= 2
         max_keys = pages * cache.page_size
         if self.window:
-            max_keys = min(max_keys, self.window + cache.page_size)
+            max_keys = min(max_keys, self.window + self.keep_first + cache.page_size)
         if self.chunk:
             max_keys = min(max_keys, self.chunk)
         nslices = K.attn_decode_slices(count, self.kv_heads, self.heads, self.head_dim, q.dtype, max_keys)
         part = ctx.buf("attn.part", (n * self.heads * nslices * (self.head_dim + 2),), torch.float32)
         K.attn_decode(q, out, part, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
                       cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,
-                      self.scale, nslices, token_list, count, slopes=self.slopes, chunk=self.chunk, sink=self.sink)
+                      self.scale, nslices, token_list, count, slopes=self.slopes, chunk=self.chunk, sink=self.sink,
+                      keep_first=self.keep_first)
 
 
 @register_part("mixer", "attention_keys_as_values")

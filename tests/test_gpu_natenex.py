@@ -141,6 +141,117 @@ def test_scaled_sum_and_scaled_embedding():
     assert torch.equal(x.cpu(), table[ids.long()] * 2.5)
 
 
+KEPT_CASES = [  # H, KV, hd, window, keep_first
+    (4, 2, 32, 24, 3), (4, 1, 64, 16, 16), (6, 2, 64, 48, 4), (2, 2, 128, 130, 17), (4, 4, 128, 32, 1), (8, 2, 96, 70, 40),
+    (2, 1, 64, 100, 70)]
+
+
+@pytest.mark.parametrize("H,KV,hd,window,keep", KEPT_CASES)
+def test_kept_first_positions_in_the_attention_kernels(H, KV, hd, window, keep):
+    """Random queries over a cache filled by hand (pages in a shuffled order; the pages between the
+    kept positions and the window hold NaN, as pages that were given back may): the kernel that
+    takes every size against a plain softmax over the keys a query sees, then the kernels on the
+    matrix cores for single tokens (in 1, 4 and 8 slices) and for prompts in blocks (a whole
+    prompt, and portions that start in the middle) against it."""
+    from kllm_amd import kernels as K
+    page, G = 16, H // KV
+    g = torch.Generator().manual_seed(H * 100 + hd + window)
+    lengths = [333, 41]
+    scale = 1.4 / hd ** 0.5
+    need = [-(-n // page) for n in lengths]
+    order = torch.randperm(sum(need) + 2, generator=g).tolist()
+    table = torch.zeros(2, max(need), dtype=torch.int32)
+    pages = torch.zeros(sum(need) + 2, 2, KV, page * hd)
+    ks, vs, qs = [], [], []
+    for s, n in enumerate(lengths):
+        k, v = torch.randn(n, KV, hd, generator=g), torch.randn(n, KV, hd, generator=g)
+        qs.append(torch.randn(n, H, hd, generator=g))
+        k, v = k.to(torch.bfloat16).float(), v.to(torch.bfloat16).float()
+        ks.append(k)
+        vs.append(v)
+        for j in range(need[s]):
+            pg = order.pop()
+            table[s, j] = pg
+            rows = slice(j * page, min((j + 1) * page, n))
+            cnt = rows.stop - rows.start
+            kk = torch.zeros(page, KV, hd)
+            vv = torch.zeros(page, KV, hd)
+            kk[:cnt], vv[:cnt] = k[rows], v[rows]
+            pages[pg, 0] = kk.permute(1, 0, 2).reshape(KV, page * hd)          # keys [slot][hd]
+            pages[pg, 1] = vv.permute(1, 2, 0).reshape(KV, hd * page)          # values [hd][slot]
+    q = torch.cat(qs).to(torch.bfloat16)
+
+    def plain(first_query):
+        out = []
+        for s, n in enumerate(lengths):
+            qq, k, v = qs[s].to(torch.bfloat16).double(), ks[s].double(), vs[s].double()
+            for i in range(first_query[s], n):
+                seen = [j for j in range(i + 1) if i - j < window or j < keep]
+                row = []
+                for h in range(H):
+                    sc = (k[seen, h // G] @ qq[i, h]) * scale
+                    row.append(torch.softmax(sc, 0) @ v[seen, h // G])
+                out.append(torch.cat(row))
+        return torch.stack(out)
+
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    want = plain([0, 0])
+    cache = pages.to("cuda", torch.bfloat16)
+    tab = table.cuda()
+    positions = i32(list(range(lengths[0])) + list(range(lengths[1])))
+    span_of = i32([0] * lengths[0] + [1] * lengths[1])
+    qd, n = q.reshape(-1, H * hd).cuda(), sum(lengths)
+    out = torch.empty(n, H * hd, device="cuda", dtype=torch.bfloat16)
+    K.attn_generic(qd, out, cache, positions, span_of, tab, page, H, KV, hd, window, scale, keep_first=keep)
+    assert rel(out.float().cpu(), want) < 1e-2
+    K.attn_generic(qd, out, cache, positions, span_of, tab, page, H, KV, hd, window, scale, keep_first=max(keep - 1, 0))
+    assert rel(out.float().cpu(), want) > 2e-2                       # one kept position fewer shows
+    # pages that lie wholly between the kept positions and the window of the LAST tokens are gone
+    holes = cache.clone()
+    for s, nl in enumerate(lengths):
+        for j in range(need[s]):
+            if j * page >= keep and (j + 1) * page <= nl - 8 - window + 1:
+                holes[table[s, j]] = float("nan")
+    last = [lengths[0] - 8, lengths[1] - 8]
+    rows_last = list(range(last[0], lengths[0])) + list(range(lengths[0] + last[1], n))
+    for nslices in (1, 4, 8):
+        out = torch.zeros(n, H * hd, device="cuda", dtype=torch.bfloat16)
+        part = torch.empty(n * H * nslices * (hd + 2), device="cuda")
+        K.attn_decode(qd, out, part, cache, positions, span_of, tab, page, H, KV, hd, window, scale, nslices, keep_first=keep)
+        assert rel(out.float().cpu(), want) < 1e-2, nslices
+        tl = i32(rows_last)
+        out.zero_()
+        K.attn_decode(qd, out, part, holes, positions, span_of, tab, page, H, KV, hd, window, scale, nslices, tl, len(rows_last),
+                      keep_first=keep)
+        assert rel(out.float().cpu()[rows_last], want[rows_last]) < 1e-2, nslices
+    if hd not in K.PREFILL_HEAD_DIMS:
+        return
+    span_start, span_pos = i32([0, lengths[0], n]), i32([0, 0])
+    tiles = [[t, 0] for t in range(0, lengths[0], K.PREFILL_QUERY_BLOCK)] + [[lengths[0], 1]]
+    for total, longest in ((0, 0), (10 ** 9, 10 ** 6), (1, 1)):          # every choice of the prompt kernel
+        out = torch.zeros(n, H * hd, device="cuda", dtype=torch.bfloat16)
+        K.attn_prefill(qd, out, cache, i32(tiles), len(tiles), span_start, span_pos, tab, page, H, KV, hd, window, scale,
+                       total, longest, keep_first=keep)
+        got = out.float().cpu()
+        for i in range(n):
+            assert rel(got[i], want[i]) < 2e-2, (total, longest, i)
+    # portions that start in the middle: the last 150 and 9 tokens, then the last 8 behind pages that are gone
+    for firsts, pool in (([lengths[0] - 150, lengths[1] - 9], cache), (last, holes)):
+        lens = [lengths[0] - firsts[0], lengths[1] - firsts[1]]
+        rows = list(range(firsts[0], lengths[0])) + list(range(lengths[0] + firsts[1], n))
+        qp = qd[rows].contiguous()
+        m = len(rows)
+        span_start, span_pos = i32([0, lens[0], m]), i32(firsts)
+        tiles = [[t, 0] for t in range(0, lens[0], K.PREFILL_QUERY_BLOCK)] + [[lens[0], 1]]
+        for total, longest in ((0, 0), (10 ** 9, 10 ** 6), (1, 1)):
+            out = torch.zeros(m, H * hd, device="cuda", dtype=torch.bfloat16)
+            K.attn_prefill(qp, out, pool, i32(tiles), len(tiles), span_start, span_pos, tab, page, H, KV, hd, window, scale,
+                           total, longest, keep_first=keep)
+            got = out.float().cpu()
+            for r, i in enumerate(rows):
+                assert rel(got[r], want[i]) < 2e-2, (firsts, total, longest, i)
+
+
 # ----------------------------------------------------------------------------- each mixer alone
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -178,7 +289,7 @@ def test_one_mixer_alone_whole_and_token_by_token(folders, name, dtype):
 # ----------------------------------------------------------------------------- aimed queries
 
 T.CONFIGS["A1"] = T._cfg(80, 64, 1e-5, 2.0, [
-    T.parallel(T.attn(4, 2, 32, rot=16, base=5000.0, scaling=(4.0, 1.0, 3.0, 48), window=24, keep=3, scale=0.45), 48, 3, 4,
+    T.parallel(T.attn(4, 2, 32, rot=16, base=5000.0, scaling=(4.0, 1.0, 3.0, 48), window=24, keep=3, scale=0.3), 48, 3, 4,
                right_scale=0.3, ff=72),
     T.delta(2, 1, 16, 24, 3)])
 T.CONFIGS["A2"] = T._cfg(96, 96, 1e-6, 1.5, [
@@ -353,6 +464,19 @@ def test_long_decoding_over_page_and_window_borders(folders, name, dtype):
     rows, rep = replay(d, dtype, steps, traces.peak_tokens(steps))
     compare(rows, expected(d, cfg, reqs, dtype), dtype, reqs)
     assert rep.engine.steps_repeated > 100                       # decode steps ran from their recorded commands
+
+
+@pytest.mark.parametrize("name", ["N5", "N6", "N7", "A3"])
+def test_the_kernel_for_every_size_and_the_matrix_core_kernels_agree(folders, name):
+    """Kept first positions behind a window in the attention kernels on the matrix cores (prompts
+    in blocks, single tokens in slices) against the kernel that takes every size, same trace."""
+    cfg, d = T.CONFIGS[name], folders(name)
+    reqs = make_requests(cfg, [300, 21, 150], 9)
+    steps, peak = traces.mixed(reqs, seed=2, max_live=3, tail=40, max_portion=70)
+    a, _ = replay(d, "bfloat16", steps, peak)
+    b, _ = replay(d, "bfloat16", steps, peak, attention="generic")
+    assert max(rel(a[k], b[k]) for k in a) < 3e-2
+    assert any(not np.array_equal(a[k], b[k]) for k in a)          # they are two kernels
 
 
 def test_recorded_steps_and_layers_change_no_bit(folders):
