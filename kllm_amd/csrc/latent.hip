@@ -13,7 +13,14 @@
 //
 // Scores, softmax, norms and rotation are 32-bit; the cached rows, the folded queries and the
 // attended latents are stored in the compute type.
+//
+// A page holds its slots' rows [slot][rank + dr] and then the latents once more, transposed
+// [rank][slot]: the weighted sum over the keys runs along the slots, and the matrix cores want
+// the dimension that is summed over contiguous.  attn_latent has two kernels: one workgroup a
+// (token, head) in 32-bit arithmetic for every size and type, and, in bfloat16 for ranks in
+// steps of 16 and rows in steps of 8, one on the matrix cores (below).
 #include <math.h>
+#include <stdint.h>
 
 #include "common.hpp"
 #include "kllm_kernels.h"
@@ -37,7 +44,10 @@ __global__ __launch_bounds__(kLatThreads) void latent_kv_append_kernel(
   const float* in = dkv + t * in_stride;
   const int pos = positions[t];
   const long page = block_table[(long)span_of_token[t] * max_pages + pos / page_size];
-  T* dst = cache + (page * page_size + pos % page_size) * row;
+  const long page_elems = (long)page_size * (row + rank);
+  const int slot = pos % page_size;
+  T* dst = cache + page * page_elems + (long)slot * row;
+  T* dst_t = cache + page * page_elems + (long)page_size * row + slot;     // [rank][slot]
   float v[kLatMaxPer];
   float ss = 0.f;
 #pragma unroll
@@ -53,7 +63,11 @@ __global__ __launch_bounds__(kLatThreads) void latent_kv_append_kernel(
 #pragma unroll
   for (int q = 0; q < kLatMaxPer; ++q) {
     const int i = tid + q * kLatThreads;
-    if (i < rank) dst[i] = from_f32<T>(v[q] * rstd * weight[i]);
+    if (i < rank) {
+      const T c = from_f32<T>(v[q] * rstd * weight[i]);
+      dst[i] = c;
+      dst_t[(long)i * page_size] = c;
+    }
   }
   for (int i = tid; i < half; i += kLatThreads) {
     float a = 0.f, b = 0.f;
@@ -132,6 +146,7 @@ __global__ __launch_bounds__(kLatThreads) void attn_latent_kernel(
   __shared__ float ps[kLatThreads];
   __shared__ float red[16];
   const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const long page_elems = (long)page_size * (row + rank);
   const int len = positions[t] + 1;
   const int* table = block_table + (long)span_of_token[t] * max_pages;
   const T* qrow = q + ((long)t * H + h) * row;
@@ -145,7 +160,7 @@ __global__ __launch_bounds__(kLatThreads) void attn_latent_kernel(
     const int key = base + tid;
     float s = -INFINITY;
     if (key < len) {
-      const T* krow = cache + ((long)table[key / page_size] * page_size + key % page_size) * row;
+      const T* krow = cache + (long)table[key / page_size] * page_elems + (long)(key % page_size) * row;
       float dot = 0.f;
       for (int i = 0; i < row; ++i) dot = fmaf(qs[i], to_f32(krow[i]), dot);
       s = dot * scale;
@@ -169,7 +184,7 @@ __global__ __launch_bounds__(kLatThreads) void attn_latent_kernel(
           const int kk = base + k;
           if (kk / page_size != pg) {
             pg = kk / page_size;
-            prow = cache + (long)table[pg] * page_size * row;
+            prow = cache + (long)table[pg] * page_elems;
           }
           a = fmaf(ps[k], to_f32(prow[(long)(kk % page_size) * row + e]), a);
         }
@@ -183,6 +198,174 @@ __global__ __launch_bounds__(kLatThreads) void attn_latent_kernel(
     const int e = tid + c * kLatThreads;
     if (e < rank) out[((long)t * H + h) * rank + e] = from_f32<T>(acc[c] / l);
   }
+}
+
+// attn_latent on the matrix cores (bfloat16).  A workgroup takes one token and up to 16 heads;
+// its four waves take the token's keys in tiles of 32, round robin, and meet in LDS.  All heads
+// read the same keys, so the 16 heads are the columns of one product:
+// MFMA 16x16x32 (lane l: g = l/16, c = l%16): A[c][8g..8g+7], B[8g..8g+7][c], D[4g+i][c].
+// Scores: A = 16 keys x 32 elements of their rows (one row per lane, straight from the page),
+// B = the folded queries of the 16 heads, D[key 4g+i][head c].  Weighted sum: the 32 slots that
+// are summed over are the keys (4g+j) of the tile's first half for j < 4 and of its second half for
+// j >= 4, which is how a lane holds its probabilities; A = latents [element c][those keys], two
+// 8-byte reads from the transposed copy.  NR: 16-element pieces of the latent a lane accumulates.
+constexpr int kLatWaves = 4;
+
+template <int NR>
+__global__ __launch_bounds__(64 * kLatWaves) void attn_latent_mfma_kernel(
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
+    const int* __restrict__ positions, const int* __restrict__ span_of_token, const int* __restrict__ block_table,
+    int max_pages, int page_size, int H, int row, int rank, float scale) {
+  extern __shared__ float lat_red[];            // [kLatWaves - 1][NR * 4 + 2][64]
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int g = lane / 16, c = lane % 16;
+  const int t = blockIdx.x, h0 = blockIdx.y * 16;
+  const int head = min(h0 + c, H - 1);
+  const bool head_ok = h0 + c < H;
+  const int len = positions[t] + 1;
+  const int* table = block_table + (long)span_of_token[t] * max_pages;
+  const long page_elems = (long)page_size * (row + rank);
+  const int ksteps = (row + 31) / 32, nr = rank / 16;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const bf16_t* qrow = q + ((long)t * H + head) * row;
+
+  float m = -INFINITY, l = 0.f;
+  floatx4 acc[NR];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) acc[r] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int tiles = (len + 31) / 32;
+  for (int tile = wave; tile < tiles; tile += kLatWaves) {
+    const int kb = tile * 32;
+    // a half (16 keys) lies in one page (pages hold a multiple of 16 slots)
+    const bf16_t* pbase[2];
+    int slot0[2];
+    bool live[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int k0 = kb + 16 * u;
+      live[u] = k0 < len;
+      const int page = table[live[u] ? k0 / page_size : 0];
+      pbase[u] = cache + (long)page * page_elems;
+      slot0[u] = live[u] ? k0 % page_size : 0;
+    }
+    floatx4 s[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
+    for (int ks = 0; ks < ksteps; ++ks) {
+      const int d0 = 32 * ks + 8 * g;
+      const bool in = d0 < row;
+      const bf16x8 qb = (in && head_ok) ? *reinterpret_cast<const bf16x8*>(qrow + d0) : zero8;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const bf16x8 a = (in && live[u]) ? *reinterpret_cast<const bf16x8*>(pbase[u] + (long)(slot0[u] + c) * row + d0) : zero8;
+        s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb, s[u], 0, 0, 0);
+      }
+    }
+    // ---- online softmax for this lane's head over its 8 keys, then over the 4 lanes of the column
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = kb + 16 * u + 4 * g + i;
+        s[u][i] = key < len ? s[u][i] * scale : -INFINITY;
+        tmax = fmaxf(tmax, s[u][i]);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+    const float m_new = fmaxf(m, tmax);                    // finite: every tile holds a key that is read
+    const float alpha = expf(m - m_new);
+    bf16x8 pb;
+    float psum = 0.f;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = (s[u][i] == -INFINITY) ? 0.f : expf(s[u][i] - m_new);
+        const bf16_t pr = (bf16_t)p;
+        pb[4 * u + i] = pr;
+        psum += (float)pr;
+      }
+    l = l * alpha + psum;
+    m = m_new;
+    // ---- the weighted sum of the latents: slots beyond the last key may hold anything
+    const bf16_t* vt[2] = {pbase[0] + (long)page_size * row + slot0[0] + 4 * g,
+                           pbase[1] + (long)page_size * row + slot0[1] + 4 * g};
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      if (r < nr) {
+        acc[r] *= alpha;
+        bf16x8 a;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const bf16x4 v = live[u] ? *reinterpret_cast<const bf16x4*>(vt[u] + (long)(16 * r + c) * page_size) : bf16x4{0, 0, 0, 0};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) a[4 * u + i] = (kb + 16 * u + 4 * g + i < len) ? v[i] : (bf16_t)0.f;
+        }
+        acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[r], 0, 0, 0);
+      }
+    }
+  }
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+
+  // ---- the waves meet: waves 1.. leave maximum, sum and output in LDS (lane-contiguous), wave 0
+  // adds them in a fixed order with weights exp(m_w - max m) and writes.
+  constexpr int kRows = NR * 4 + 2;
+  if (wave > 0) {
+    float* mine = lat_red + (long)(wave - 1) * kRows * kWave + lane;
+#pragma unroll
+    for (int r = 0; r < NR; ++r)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mine[(4 * r + i) * kWave] = acc[r][i];
+    mine[(NR * 4) * kWave] = m;
+    mine[(NR * 4 + 1) * kWave] = l;
+  }
+  __syncthreads();
+  if (wave > 0 || !head_ok) return;
+  float mw[kLatWaves - 1], ww[kLatWaves - 1], M = m;
+#pragma unroll
+  for (int w = 0; w < kLatWaves - 1; ++w) {
+    mw[w] = lat_red[((long)w * kRows + NR * 4) * kWave + lane];
+    M = fmaxf(M, mw[w]);
+  }
+  const float w0 = expf(m - M);                             // wave 0 holds key 0: M is finite
+  l *= w0;
+#pragma unroll
+  for (int w = 0; w < kLatWaves - 1; ++w) {
+    ww[w] = (mw[w] == -INFINITY) ? 0.f : expf(mw[w] - M);
+    l += ww[w] * lat_red[((long)w * kRows + NR * 4 + 1) * kWave + lane];
+  }
+  const float inv = 1.f / l;
+  bf16_t* orow = out + ((long)t * H + head) * rank;
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    if (r < nr) {
+      bf16x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float o = acc[r][i] * w0;
+#pragma unroll
+        for (int w = 0; w < kLatWaves - 1; ++w) o += ww[w] * lat_red[((long)w * kRows + 4 * r + i) * kWave + lane];
+        v[i] = (bf16_t)(o * inv);
+      }
+      *reinterpret_cast<bf16x4*>(orow + 16 * r + 4 * g) = v;
+    }
+  }
+}
+
+template <int NR>
+static void launch_latent_mfma(const void* q, void* out, const void* cache, const int* positions, const int* span_of_token,
+                               const int* block_table, int max_pages, int page_size, int n, int H, int row, int rank,
+                               float scale, hipStream_t stream) {
+  const size_t lds = (size_t)(kLatWaves - 1) * (NR * 4 + 2) * kWave * sizeof(float);
+  static int raised = 0;
+  if (lds > 64 * 1024 && !raised) {
+    (void)hipFuncSetAttribute((const void*)attn_latent_mfma_kernel<NR>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    raised = 1;
+  }
+  hipLaunchKernelGGL(attn_latent_mfma_kernel<NR>, dim3(n, (H + 15) / 16), dim3(64 * kLatWaves), lds, stream,
+                     (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, positions, span_of_token, block_table, max_pages,
+                     page_size, H, row, rank, scale);
 }
 
 // attended: [n][H][rank]; w_uv [H * dv][rank]; gate: [nsplit][n][H * dv] sums or null.
@@ -273,12 +456,20 @@ extern "C" int kllm_latent_query(const float* q, int nsplit, long split_stride, 
 
 extern "C" int kllm_attn_latent(const void* q, void* out, const void* cache, const int* positions,
                                 const int* span_of_token, const int* block_table, int max_pages, int page_size, int n,
-                                int H, int row, int rank, float scale, int dtype, hipStream_t stream) {
+                                int H, int row, int rank, float scale, int dtype, int mode, hipStream_t stream) {
   KLLM_REQUIRE(q && out && cache && positions && span_of_token && block_table, "attn_latent: null pointer");
   KLLM_REQUIRE(n > 0 && H > 0 && H <= 65535 && rank > 0 && rank <= row && row <= kLatMaxRow,
                "attn_latent: bad sizes n=%d H=%d row=%d rank=%d (rows of up to %d)", n, H, row, rank, kLatMaxRow);
   KLLM_REQUIRE(max_pages > 0 && page_size > 0, "attn_latent: bad cache sizes");
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "attn_latent: unknown dtype %d", dtype);
+  if (dtype == DT_BF16 && mode != 1 && rank % 16 == 0 && row % 8 == 0 && rank <= 512 && page_size % 16 == 0 &&
+      ((uintptr_t)q & 15) == 0 && ((uintptr_t)cache & 15) == 0 && ((uintptr_t)out & 7) == 0) {
+    if (rank <= 128) launch_latent_mfma<8>(q, out, cache, positions, span_of_token, block_table, max_pages, page_size, n, H, row, rank, scale, stream);
+    else if (rank <= 256) launch_latent_mfma<16>(q, out, cache, positions, span_of_token, block_table, max_pages, page_size, n, H, row, rank, scale, stream);
+    else launch_latent_mfma<32>(q, out, cache, positions, span_of_token, block_table, max_pages, page_size, n, H, row, rank, scale, stream);
+    KLLM_CHECK_LAUNCH("attn_latent");
+    return 0;
+  }
   if (dtype == DT_F32)
     hipLaunchKernelGGL(attn_latent_kernel<float>, dim3(n, H), dim3(kLatThreads), 0, stream, (const float*)q,
                        (float*)out, (const float*)cache, positions, span_of_token, block_table, max_pages, page_size, H,

@@ -159,7 +159,7 @@ def _declare(lib):
         "kllm_latent_kv_append": [P, I, L, P, F, P, P, P, P, P, P, I, I, I, I, I, I, L, P],
         "kllm_latent_norm": [P, I, L, L, P, F, P, I, I, I, P],
         "kllm_latent_query": [P, I, L, P, P, P, P, I, I, I, I, I, I, P],
-        "kllm_attn_latent": [P, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
+        "kllm_attn_latent": [P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "kllm_latent_out": [P, P, P, I, L, L, P, I, I, I, I, I, P],
     }
     for name, args in sigs.items():
@@ -1705,11 +1705,12 @@ def latent_kv_append(sums, first_column, weight, eps, cos, sin, cache, positions
                      rank, rot_dim):
     """Columns first_column .. + rank + rot_dim of the float32 sums: the first ``rank`` through an RMS
     norm with ``weight``, the rest rotated (halves paired; cos, sin [n, rot_dim / 2]); the row is
-    appended to the pages (``cache`` [pages, page_size * (rank + rot_dim)])."""
+    appended to the pages (``cache`` [pages, page_size * (rank + rot_dim) + rank * page_size]: a
+    page's rows, then the normalised part once more as [rank][slot])."""
     n = cos.shape[0]
     row = rank + rot_dim
     addr, nsplit, stride, cols = _columns(sums, first_column, row, "latent_kv_append")
-    if (sums.shape[-2] != n or cache.dim() != 2 or cache.shape[1] != page_size * row or weight.numel() != rank
+    if (sums.shape[-2] != n or cache.dim() != 2 or cache.shape[1] != page_size * (row + rank) or weight.numel() != rank
             or tuple(cos.shape) != (n, rot_dim // 2) or tuple(sin.shape) != tuple(cos.shape)
             or positions.numel() < n or span_of_token.numel() < n):
         raise KernelError("latent_kv_append: shapes do not fit")
@@ -1746,12 +1747,14 @@ def latent_query(q, w_uk, cos, sin, out, heads, dim, rot_dim, rank):
             int(dim), int(rot_dim), int(rank), dtype_code(out.dtype), _stream())
 
 
-def attn_latent(q, out, cache, positions, span_of_token, block_table, page_size, heads, row, rank, scale):
+def attn_latent(q, out, cache, positions, span_of_token, block_table, page_size, heads, row, rank, scale, plain=False):
     """Causal attention of q [n, H row] over cached rows of ``row`` elements whose first ``rank``
-    are also the values: out [n, H rank]."""
+    are also the values (a page: its rows, then the first ``rank`` elements once more as
+    [rank][slot]): out [n, H rank].  ``plain``: the kernel for every size, also where the one on
+    the matrix cores fits."""
     n = q.shape[0]
     if (tuple(q.shape) != (n, heads * row) or tuple(out.shape) != (n, heads * rank) or q.dtype != cache.dtype
-            or out.dtype != q.dtype or cache.dim() != 2 or cache.shape[1] != page_size * row
+            or out.dtype != q.dtype or cache.dim() != 2 or cache.shape[1] != page_size * (row + rank)
             or positions.numel() < n or span_of_token.numel() < n):
         raise KernelError("attn_latent: shapes or dtypes do not fit")
     I32 = torch.int32
@@ -1759,7 +1762,7 @@ def attn_latent(q, out, cache, positions, span_of_token, block_table, page_size,
             _ptr(cache, "attn_latent cache"), _ptr(positions, "attn_latent positions", I32),
             _ptr(span_of_token, "attn_latent span_of_token", I32), _ptr(block_table, "attn_latent block_table", I32),
             block_table.shape[1], int(page_size), n, int(heads), int(row), int(rank), float(scale), dtype_code(q.dtype),
-            _stream())
+            int(bool(plain)), _stream())
 
 
 def latent_out(attended, w_uv, out, heads, vdim, rank, gate=None, gate_column=0):

@@ -8,8 +8,9 @@ W_uv,h c; the score is (q . k) * ``scale`` over all ``head_dim`` + ``rot_dim`` e
 over the positions up to the query's; the concatenated heads are multiplied by sigmoid(W_g h)
 and projected by W_o.
 
-Only c and the rotated part are cached: one row of ``kv_rank`` + ``rot_dim`` a token (a paged
-cache with one "head" and no values).  The products with W_uk and W_uv are moved to the other
+Only c and the rotated part are cached: one row of ``kv_rank`` + ``rot_dim`` a token, and c once
+more with the slots of a page side by side (a paged cache with one "head" whose "values" are
+c: the weighted sum over the keys runs along the slots).  The products with W_uk and W_uv are moved to the other
 side: the query's unrotated part is folded through W_uk,h once a token, so that the score is
 taken against c itself; the softmax's weighted sum is taken of c, and W_uv,h is applied to that
 sum.  The numbers are the ones of the definition up to rounding.
@@ -86,7 +87,7 @@ class LatentAttention(Part):
         return [self.w_in, self.w_uq, self.w_uk, self.w_uv, self.w_o, self.q_norm, self.kv_norm]
 
     def cache_need(self):
-        return CacheNeed("paged", kv_heads=1, head_dim=self.row, value_dim=0)
+        return CacheNeed("paged", kv_heads=1, head_dim=self.row, value_dim=self.kv_rank)
 
     def check_cache(self, page_size):
         if self.row > K.latent_max_row():
@@ -112,7 +113,8 @@ class LatentAttention(Part):
         K.latent_query(q, self.w_uk, cos, sin, qa, self.heads, self.head_dim, self.rot_dim, self.kv_rank)
         attended = ctx.buf("latent.att", (n, self.heads * self.kv_rank), dtype)
         K.attn_latent(qa, attended, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table, cache.page_size,
-                      self.heads, self.row, self.kv_rank, self.scale)
+                      self.heads, self.row, self.kv_rank, self.scale,
+                      plain=self.runtime.options.get("attention", "auto") == "generic")
         out = ctx.buf("latent.out", (n, self.out_dim), dtype)
         K.latent_out(attended, self.w_uv, out, self.heads, self.value_dim, self.kv_rank,
                      gate=first if self.gated else None, gate_column=self.q_rank + self.row)

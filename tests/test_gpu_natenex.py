@@ -26,8 +26,9 @@ pytestmark = pytest.mark.gpu
 DTYPES = ["float32", "bfloat16"]
 F64 = torch.float64
 # Logits: root mean square of the difference (mean taken off) over that of the plain model's logits.
-# In bfloat16 a position's limit is three times what rounding of the sub-layers' inputs alone does
-# to the plain model there, where that is more.  Measured over this file: float32 at most 4e-6;
+# In bfloat16 a position's limit is five times what rounding of the sub-layers' inputs alone does
+# to the plain model there, where that is more (the engine also keeps queries, keys, values,
+# probabilities and the activations inside a mixer in bfloat16).  Measured over this file: float32 at most 4e-6;
 # bfloat16 at most 4.9e-2, at an aimed query whose scores reach 17 (queries and keys are kept in
 # bfloat16, which moves such a score by several hundredths), with a median near 1e-2.
 TOL = {"float32": 2e-5, "bfloat16": 6e-2}
@@ -116,8 +117,8 @@ def compare(rows, want, dtype, requests, tol=None):
             assert np.isfinite(got).all(), (rid, p)
             err = row_error(got, want[rid][p])
             limit = tol or TOL[dtype]
-            if getattr(want, "slack", None):      # three times what rounding alone does there, if that is more
-                limit = max(limit, 3.0 * want.slack[rid][p])
+            if getattr(want, "slack", None):      # five times what rounding of the inputs alone does there, if that is more
+                limit = max(limit, 5.0 * want.slack[rid][p])
             worst = max(worst, err * (tol or TOL[dtype]) / limit)
             assert err < limit, f"{rid} position {p}: off by {err} (limit {limit})"
     assert len(rows) == sum(len(t) for t in requests.values())
@@ -252,6 +253,69 @@ def test_kept_first_positions_in_the_attention_kernels(H, KV, hd, window, keep):
                 assert rel(got[r], want[i]) < 2e-2, (firsts, total, longest, i)
 
 
+LATENT_CASES = [(3, 40, 8), (6, 160, 32), (3, 448, 64), (20, 96, 32), (34, 128, 16), (2, 512, 64), (5, 200, 24), (4, 16, 8)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,rank,dr", LATENT_CASES)
+def test_attention_over_cached_latents(H, rank, dr, dtype):
+    """Folded queries over rows appended by the framework's own kernel (pages in a shuffled
+    order, what lies behind a request's last token is NaN): the kernel for every size and, where
+    it fits, the one on the matrix cores against a plain softmax over the rows, whose first
+    ``rank`` elements are the values; one query looks along a key hundreds of positions back."""
+    from kllm_amd import kernels as K
+    dt = {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype]
+    page, row, eps = 16, rank + dr, 1e-5
+    g = torch.Generator().manual_seed(H * 1000 + rank)
+    lengths = [431, 19]
+    scale = 1.2 / row ** 0.5
+    need = [-(-n // page) for n in lengths]
+    order = torch.randperm(sum(need) + 2, generator=g).tolist()
+    table = torch.zeros(2, max(need), dtype=torch.int32)
+    for s in range(2):
+        for j in range(need[s]):
+            table[s, j] = order.pop()
+    n = sum(lengths)
+    sums = torch.randn(2, n, row + 5, generator=g)          # two slices of a product, the rows start at column 5
+    weight = 1.0 + 0.2 * torch.randn(rank, generator=g)
+    positions = list(range(lengths[0])) + list(range(lengths[1]))
+    span_of = [0] * lengths[0] + [1] * lengths[1]
+    rot = {"dims": dr, "base": 700.0}
+    raw = sums.double().sum(0)[:, 5:]
+    rows = torch.cat([P.rms_norm(raw[:, :rank], weight.double(), eps),
+                      torch.cat([P.rotate_halves(raw[a:a + 1, None, rank:], [positions[a]], rot)[:, 0] for a in range(n)])], dim=1)
+    q = torch.randn(n, H, row, generator=g)
+    q[400, :, :rank] = 6.0 * rows[3, :rank].float() / rows[3, :rank].norm().float() * row ** 0.5 / 1.2   # looks along key 3
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    cache = torch.full((sum(need) + 2, page * (row + rank)), float("nan"), device="cuda", dtype=dt)
+    freq = P.frequencies(rot)
+    cos, sin = torch.empty(n, dr // 2, device="cuda"), torch.empty(n, dr // 2, device="cuda")
+    K.rope_tables_freq(cos, sin, i32(positions), freq.cuda(), 1.0)
+    K.latent_kv_append(sums.cuda(), 5, weight.cuda(), eps, cos, sin, cache, i32(positions), i32(span_of), table.cuda(), page,
+                       rank, dr)
+    stored = rows.to(dt).double()
+    qd = q.reshape(n, H * row).to("cuda", dt)
+    qq = qd.cpu().double().reshape(n, H, row)
+    want = torch.zeros(n, H, rank, dtype=F64)
+    base = 0
+    for s, nl in enumerate(lengths):
+        kk = stored[base:base + nl]
+        for i in range(nl):
+            sc = torch.einsum("hd,kd->hk", qq[base + i], kk[:i + 1]) * scale
+            want[base + i] = torch.softmax(sc, -1) @ kk[:i + 1, :rank]
+        base += nl
+    assert float(torch.softmax(torch.einsum("hd,kd->hk", qq[400], stored[:401]) * scale, -1)[:, 3].min()) > 0.5
+    tol = 2e-5 if dtype == "float32" else 1.5e-2
+    for plain in (True, False):
+        out = torch.zeros(n, H * rank, device="cuda", dtype=dt)
+        K.attn_latent(qd, out, cache, i32(positions), i32(span_of), table.cuda(), page, H, row, rank, scale, plain=plain)
+        got = out.float().cpu().reshape(n, H, rank)
+        assert torch.isfinite(got).all()
+        for i in (0, 1, 15, 16, 17, 400, 430, 431, 449):
+            assert rel(got[i], want[i]) < tol, (plain, i)
+        assert rel(got, want) < tol, plain
+
+
 # ----------------------------------------------------------------------------- each mixer alone
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -289,7 +353,7 @@ def test_one_mixer_alone_whole_and_token_by_token(folders, name, dtype):
 # ----------------------------------------------------------------------------- aimed queries
 
 T.CONFIGS["A1"] = T._cfg(80, 64, 1e-5, 2.0, [
-    T.parallel(T.attn(4, 2, 32, rot=16, base=5000.0, scaling=(4.0, 1.0, 3.0, 48), window=24, keep=3, scale=0.3), 48, 3, 4,
+    T.parallel(T.attn(4, 2, 32, rot=16, base=5000.0, scaling=(4.0, 1.0, 3.0, 48), window=24, keep=3, scale=0.2), 48, 3, 4,
                right_scale=0.3, ff=72),
     T.delta(2, 1, 16, 24, 3)])
 T.CONFIGS["A2"] = T._cfg(96, 96, 1e-6, 1.5, [
