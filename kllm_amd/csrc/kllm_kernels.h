@@ -469,10 +469,10 @@ int kllm_latent_norm(const float* in, int nsplit, long split_stride, long in_str
                      void* out, int n, int r, int dtype, hipStream_t stream);
 int kllm_latent_query(const float* q, int nsplit, long split_stride, const void* w_uk, const float* cos_t,
                       const float* sin_t, void* out, int n, int H, int d, int dr, int rank, int dtype,
-                      hipStream_t stream);
+                      int transposed, hipStream_t stream);
 int kllm_attn_latent(const void* q, void* out, const void* cache, const int* positions, const int* span_of_token,
                      const int* block_table, int max_pages, int page_size, int n, int H, int row, int rank,
-                     float scale, int dtype, int mode, hipStream_t stream);
+                     float scale, int dtype, int mode, float* part, long part_floats, int nslices, hipStream_t stream);
 int kllm_latent_out(const void* attended, const void* w_uv, const float* gate, int nsplit, long split_stride,
                     long gate_stride, void* out, int n, int H, int dv, int rank, int dtype, hipStream_t stream);
 

@@ -215,7 +215,7 @@ template <int NR>
 __global__ __launch_bounds__(64 * kLatWaves) void attn_latent_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ span_of_token, const int* __restrict__ block_table,
-    int max_pages, int page_size, int H, int row, int rank, float scale) {
+    int max_pages, int page_size, int H, int row, int rank, float scale, float* __restrict__ part) {
   extern __shared__ float lat_red[];            // [kLatWaves - 1][NR * 4 + 2][64]
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int g = lane / 16, c = lane % 16;
@@ -234,8 +234,11 @@ __global__ __launch_bounds__(64 * kLatWaves) void attn_latent_mfma_kernel(
 #pragma unroll
   for (int r = 0; r < NR; ++r) acc[r] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+  // The tiles go in turn to the slices (workgroups of the same token and heads, blockIdx.z: where
+  // tokens and heads alone leave CUs idle) and, within a slice, to the waves.
+  const int nslices = gridDim.z, slice = blockIdx.z;
   const int tiles = (len + 31) / 32;
-  for (int tile = wave; tile < tiles; tile += kLatWaves) {
+  for (int tile = slice * kLatWaves + wave; tile < tiles; tile += kLatWaves * nslices) {
     const int kb = tile * 32;
     // a half (16 keys) lies in one page (pages hold a multiple of 16 slots)
     const bf16_t* pbase[2];
@@ -328,12 +331,34 @@ __global__ __launch_bounds__(64 * kLatWaves) void attn_latent_mfma_kernel(
     mw[w] = lat_red[((long)w * kRows + NR * 4) * kWave + lane];
     M = fmaxf(M, mw[w]);
   }
-  const float w0 = expf(m - M);                             // wave 0 holds key 0: M is finite
+  const float w0 = (m == -INFINITY) ? 0.f : expf(m - M);    // (a slice beyond the token's keys has none)
   l *= w0;
 #pragma unroll
   for (int w = 0; w < kLatWaves - 1; ++w) {
     ww[w] = (mw[w] == -INFINITY) ? 0.f : expf(mw[w] - M);
     l += ww[w] * lat_red[((long)w * kRows + NR * 4 + 1) * kWave + lane];
+  }
+  if (nslices > 1) {
+    // the slice's sums as they are, with its maximum and its sum of probabilities: rows of
+    // rank + 2 floats; a slice without a key leaves a maximum of -inf and zeros
+    float* prow = part + (((long)t * H + head) * nslices + slice) * (rank + 2);
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      if (r < nr) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float o = acc[r][i] * w0;
+#pragma unroll
+          for (int w = 0; w < kLatWaves - 1; ++w) o += ww[w] * lat_red[((long)w * kRows + 4 * r + i) * kWave + lane];
+          prow[16 * r + 4 * g + i] = o;
+        }
+      }
+    }
+    if (g == 0) {
+      prow[rank] = M;
+      prow[rank + 1] = l;
+    }
+    return;
   }
   const float inv = 1.f / l;
   bf16_t* orow = out + ((long)t * H + head) * rank;
@@ -353,19 +378,44 @@ __global__ __launch_bounds__(64 * kLatWaves) void attn_latent_mfma_kernel(
   }
 }
 
+// The slices' results of one (token, head) become its output: weights exp(m_s - max m).
+__global__ __launch_bounds__(kLatThreads) void attn_latent_merge_kernel(const float* __restrict__ part,
+                                                                        bf16_t* __restrict__ out, int rank, int nslices) {
+  const long th = blockIdx.x;
+  const float* rows = part + th * nslices * (rank + 2);
+  float M = -INFINITY;
+  for (int s = 0; s < nslices; ++s) M = fmaxf(M, rows[(long)s * (rank + 2) + rank]);
+  float l = 0.f;
+  for (int s = 0; s < nslices; ++s) {
+    const float ms = rows[(long)s * (rank + 2) + rank];
+    if (ms != -INFINITY) l += expf(ms - M) * rows[(long)s * (rank + 2) + rank + 1];
+  }
+  const float inv = 1.f / l;
+  for (int e = threadIdx.x; e < rank; e += kLatThreads) {
+    float o = 0.f;
+    for (int s = 0; s < nslices; ++s) {
+      const float ms = rows[(long)s * (rank + 2) + rank];
+      if (ms != -INFINITY) o = fmaf(expf(ms - M), rows[(long)s * (rank + 2) + e], o);
+    }
+    out[th * rank + e] = (bf16_t)(o * inv);
+  }
+}
+
 template <int NR>
 static void launch_latent_mfma(const void* q, void* out, const void* cache, const int* positions, const int* span_of_token,
                                const int* block_table, int max_pages, int page_size, int n, int H, int row, int rank,
-                               float scale, hipStream_t stream) {
+                               float scale, float* part, int nslices, hipStream_t stream) {
   const size_t lds = (size_t)(kLatWaves - 1) * (NR * 4 + 2) * kWave * sizeof(float);
   static int raised = 0;
   if (lds > 64 * 1024 && !raised) {
     (void)hipFuncSetAttribute((const void*)attn_latent_mfma_kernel<NR>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     raised = 1;
   }
-  hipLaunchKernelGGL(attn_latent_mfma_kernel<NR>, dim3(n, (H + 15) / 16), dim3(64 * kLatWaves), lds, stream,
+  hipLaunchKernelGGL(attn_latent_mfma_kernel<NR>, dim3(n, (H + 15) / 16, nslices), dim3(64 * kLatWaves), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, positions, span_of_token, block_table, max_pages,
-                     page_size, H, row, rank, scale);
+                     page_size, H, row, rank, scale, part);
+  if (nslices > 1)
+    hipLaunchKernelGGL(attn_latent_merge_kernel, dim3(n * H), dim3(kLatThreads), 0, stream, part, (bf16_t*)out, rank, nslices);
 }
 
 // attended: [n][H][rank]; w_uv [H * dv][rank]; gate: [nsplit][n][H * dv] sums or null.
@@ -390,6 +440,97 @@ __global__ __launch_bounds__(kLatThreads) void latent_out_kernel(
       acc *= sigmoid_f32(g);
     }
     out[t * H * dv + col] = from_f32<T>(acc);
+  }
+}
+
+// The two products with a head's own matrix on the matrix cores (bfloat16), MFMA 16x16x32 as
+// above: a wave takes 16 outputs (rows of the head's matrix, one per lane, 16 bytes at a time)
+// and 16 tokens, a workgroup four such pieces of 16 outputs.
+//   latent_out:   out[t][h][j] = sum_r W_uv[h dv + j][r] attended[t][h][r], times the gate
+//   latent_query: out[t][h][r] = sum_i W_ukT[h][r][i] q[t][h][i] (W_ukT: the head's matrix
+//                 transposed once, when the weights are bound), and the rotated part beside it
+__global__ __launch_bounds__(kLatThreads) void latent_out_mfma_kernel(
+    const bf16_t* __restrict__ attended, const bf16_t* __restrict__ w_uv, const float* __restrict__ gate, int nsplit,
+    long split_stride, long gate_stride, bf16_t* __restrict__ out, int n, int H, int dv, int rank) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int g = lane / 16, c = lane % 16;
+  const int h = blockIdx.y;
+  const int j0 = (blockIdx.z * 4 + wave) * 16;
+  if (j0 >= dv) return;
+  const int t = min((int)blockIdx.x * 16 + c, n - 1);
+  const int j = min(j0 + c, dv - 1);
+  const bf16_t* wrow = w_uv + ((long)h * dv + j) * rank;
+  const bf16_t* arow = attended + ((long)t * H + h) * rank;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 8 * g; k0 < rank; k0 += 32) {            // rank % 32 == 0 (the launch): every lane takes every step
+    const bf16x8 a = *reinterpret_cast<const bf16x8*>(wrow + k0);
+    const bf16x8 b = *reinterpret_cast<const bf16x8*>(arow + k0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+  }
+  const int tt = blockIdx.x * 16 + c;
+  if (tt >= n) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int jj = j0 + 4 * g + i;
+    if (jj >= dv) continue;
+    const long col = (long)h * dv + jj;
+    float v = acc[i];
+    if (gate) {
+      float gs = 0.f;
+      for (int s = 0; s < nsplit; ++s) gs += gate[s * split_stride + tt * gate_stride + col];
+      v *= sigmoid_f32(gs);
+    }
+    out[(long)tt * H * dv + col] = (bf16_t)v;
+  }
+}
+
+__global__ __launch_bounds__(kLatThreads) void latent_query_mfma_kernel(
+    const float* __restrict__ q, int nsplit, long split_stride, const bf16_t* __restrict__ w_ukt,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, bf16_t* __restrict__ out, int n, int H, int d,
+    int dr, int rank) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int g = lane / 16, c = lane % 16;
+  const int h = blockIdx.y;
+  const int hw = d + dr, half = dr / 2;
+  const int t = min((int)blockIdx.x * 16 + c, n - 1);
+  const int tt = blockIdx.x * 16 + c;
+  const float* in = q + ((long)t * H + h) * hw;
+  const int r0 = (blockIdx.z * 4 + wave) * 16;
+  if (r0 < rank) {
+    const int r = min(r0 + c, rank - 1);
+    const bf16_t* wrow = w_ukt + ((long)h * rank + r) * d;
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 8 * g; k0 < d; k0 += 32) {               // d % 32 == 0 (the launch)
+      const bf16x8 a = *reinterpret_cast<const bf16x8*>(wrow + k0);
+      bf16x8 b;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float v = 0.f;
+        for (int s = 0; s < nsplit; ++s) v += in[s * split_stride + k0 + e];
+        b[e] = (bf16_t)v;
+      }
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+    }
+    if (tt < n) {
+      bf16_t* dst = out + ((long)tt * H + h) * (rank + dr);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (r0 + 4 * g + i < rank) dst[r0 + 4 * g + i] = (bf16_t)acc[i];
+    }
+  }
+  // the rotated part: the workgroup's first piece of outputs takes it along
+  if (blockIdx.z == 0 && wave == 0 && tt < n) {
+    bf16_t* dst = out + ((long)tt * H + h) * (rank + dr);
+    for (int i = g; i < half; i += 4) {
+      float a = 0.f, b = 0.f;
+      for (int s = 0; s < nsplit; ++s) {
+        a += in[s * split_stride + d + i];
+        b += in[s * split_stride + d + half + i];
+      }
+      const float cs = cos_t[(long)tt * half + i], sn = sin_t[(long)tt * half + i];
+      dst[rank + i] = (bf16_t)(a * cs - b * sn);
+      dst[rank + half + i] = (bf16_t)(b * cs + a * sn);
+    }
   }
 }
 
@@ -437,12 +578,20 @@ extern "C" int kllm_latent_norm(const float* in, int nsplit, long split_stride, 
 
 extern "C" int kllm_latent_query(const float* q, int nsplit, long split_stride, const void* w_uk, const float* cos_t,
                                  const float* sin_t, void* out, int n, int H, int d, int dr, int rank, int dtype,
-                                 hipStream_t stream) {
+                                 int transposed, hipStream_t stream) {
   KLLM_REQUIRE(q && w_uk && cos_t && sin_t && out, "latent_query: null pointer");
   KLLM_REQUIRE(n > 0 && nsplit >= 1 && H > 0 && H <= 65535 && d > 0 && dr > 0 && dr % 2 == 0 && rank > 0 &&
                    rank + dr <= kLatMaxRow && d + dr <= 4096,
                "latent_query: bad sizes n=%d H=%d d=%d dr=%d rank=%d", n, H, d, dr, rank);
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "latent_query: unknown dtype %d", dtype);
+  if (transposed) {     // w_uk is [H][rank][d]: the kernel on the matrix cores
+    KLLM_REQUIRE(dtype == DT_BF16 && d % 32 == 0 && ((uintptr_t)w_uk & 15) == 0,
+                 "latent_query: the transposed matrix goes with bfloat16 and head sizes in steps of 32 (d=%d)", d);
+    hipLaunchKernelGGL(latent_query_mfma_kernel, dim3((n + 15) / 16, H, (rank + 63) / 64), dim3(kLatThreads), 0, stream, q,
+                       nsplit, split_stride, (const bf16_t*)w_uk, cos_t, sin_t, (bf16_t*)out, n, H, d, dr, rank);
+    KLLM_CHECK_LAUNCH("latent_query");
+    return 0;
+  }
   const size_t lds = (size_t)(d + dr) * sizeof(float);
   if (dtype == DT_F32)
     hipLaunchKernelGGL(latent_query_kernel<float>, dim3(n, H), dim3(kLatThreads), lds, stream, q, nsplit, split_stride,
@@ -456,7 +605,8 @@ extern "C" int kllm_latent_query(const float* q, int nsplit, long split_stride, 
 
 extern "C" int kllm_attn_latent(const void* q, void* out, const void* cache, const int* positions,
                                 const int* span_of_token, const int* block_table, int max_pages, int page_size, int n,
-                                int H, int row, int rank, float scale, int dtype, int mode, hipStream_t stream) {
+                                int H, int row, int rank, float scale, int dtype, int mode, float* part, long part_floats, int nslices,
+                                hipStream_t stream) {
   KLLM_REQUIRE(q && out && cache && positions && span_of_token && block_table, "attn_latent: null pointer");
   KLLM_REQUIRE(n > 0 && H > 0 && H <= 65535 && rank > 0 && rank <= row && row <= kLatMaxRow,
                "attn_latent: bad sizes n=%d H=%d row=%d rank=%d (rows of up to %d)", n, H, row, rank, kLatMaxRow);
@@ -464,9 +614,12 @@ extern "C" int kllm_attn_latent(const void* q, void* out, const void* cache, con
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "attn_latent: unknown dtype %d", dtype);
   if (dtype == DT_BF16 && mode != 1 && rank % 16 == 0 && row % 8 == 0 && rank <= 512 && page_size % 16 == 0 &&
       ((uintptr_t)q & 15) == 0 && ((uintptr_t)cache & 15) == 0 && ((uintptr_t)out & 7) == 0) {
-    if (rank <= 128) launch_latent_mfma<8>(q, out, cache, positions, span_of_token, block_table, max_pages, page_size, n, H, row, rank, scale, stream);
-    else if (rank <= 256) launch_latent_mfma<16>(q, out, cache, positions, span_of_token, block_table, max_pages, page_size, n, H, row, rank, scale, stream);
-    else launch_latent_mfma<32>(q, out, cache, positions, span_of_token, block_table, max_pages, page_size, n, H, row, rank, scale, stream);
+    KLLM_REQUIRE(nslices >= 1 && nslices <= 64 && (nslices == 1 || (part && part_floats >= (long)n * H * nslices * (rank + 2))),
+                 "attn_latent: %d slices need room for %d tokens x %d heads x %d slices x (%d + 2) floats", nslices, n, H,
+                 nslices, rank);
+    if (rank <= 128) launch_latent_mfma<8>(q, out, cache, positions, span_of_token, block_table, max_pages, page_size, n, H, row, rank, scale, part, nslices, stream);
+    else if (rank <= 256) launch_latent_mfma<16>(q, out, cache, positions, span_of_token, block_table, max_pages, page_size, n, H, row, rank, scale, part, nslices, stream);
+    else launch_latent_mfma<32>(q, out, cache, positions, span_of_token, block_table, max_pages, page_size, n, H, row, rank, scale, part, nslices, stream);
     KLLM_CHECK_LAUNCH("attn_latent");
     return 0;
   }
@@ -489,6 +642,13 @@ extern "C" int kllm_latent_out(const void* attended, const void* w_uv, const flo
   KLLM_REQUIRE(n > 0 && H > 0 && H <= 65535 && dv > 0 && rank > 0 && rank <= 8192 && (!gate || nsplit >= 1),
                "latent_out: bad sizes n=%d H=%d dv=%d rank=%d", n, H, dv, rank);
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "latent_out: unknown dtype %d", dtype);
+  if (dtype == DT_BF16 && rank % 32 == 0 && ((uintptr_t)attended & 15) == 0 && ((uintptr_t)w_uv & 15) == 0) {
+    hipLaunchKernelGGL(latent_out_mfma_kernel, dim3((n + 15) / 16, H, (dv + 63) / 64), dim3(kLatThreads), 0, stream,
+                       (const bf16_t*)attended, (const bf16_t*)w_uv, gate, nsplit, split_stride, gate_stride, (bf16_t*)out,
+                       n, H, dv, rank);
+    KLLM_CHECK_LAUNCH("latent_out");
+    return 0;
+  }
   const size_t lds = (size_t)rank * sizeof(float);
   if (dtype == DT_F32)
     hipLaunchKernelGGL(latent_out_kernel<float>, dim3(n, H), dim3(kLatThreads), lds, stream, (const float*)attended,

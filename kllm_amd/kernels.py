@@ -158,8 +158,8 @@ def _declare(lib):
         "kllm_latent_max_row": [],
         "kllm_latent_kv_append": [P, I, L, P, F, P, P, P, P, P, P, I, I, I, I, I, I, L, P],
         "kllm_latent_norm": [P, I, L, L, P, F, P, I, I, I, P],
-        "kllm_latent_query": [P, I, L, P, P, P, P, I, I, I, I, I, I, P],
-        "kllm_attn_latent": [P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
+        "kllm_latent_query": [P, I, L, P, P, P, P, I, I, I, I, I, I, I, P],
+        "kllm_attn_latent": [P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P, L, I, P],
         "kllm_latent_out": [P, P, P, I, L, L, P, I, I, I, I, I, P],
     }
     for name, args in sigs.items():
@@ -1732,22 +1732,39 @@ def latent_norm(sums, first_column, weight, eps, out):
             float(eps), _ptr(out, "latent_norm out"), n, r, dtype_code(out.dtype), _stream())
 
 
-def latent_query(q, w_uk, cos, sin, out, heads, dim, rot_dim, rank):
+def latent_query(q, w_uk, cos, sin, out, heads, dim, rot_dim, rank, transposed=False):
     """q: float32 sums [nsplit, n, H (dim + rot_dim)], a head laid out [dim | rot_dim].  out [n, H
     (rank + rot_dim)]: per head the first dim folded through w_uk ([H dim, rank]: sum_i q_i w[i, :]),
-    then the rotated rest."""
+    then the rotated rest.  ``transposed``: w_uk is given head by head as [H rank, dim] (bfloat16,
+    dim in steps of 32): the product runs on the matrix cores."""
     n = out.shape[0]
     nsplit, stride = _splits(q, n, heads * (dim + rot_dim), "latent_query")
-    if (tuple(out.shape) != (n, heads * (rank + rot_dim)) or tuple(w_uk.shape) != (heads * dim, rank)
+    if (tuple(out.shape) != (n, heads * (rank + rot_dim))
+            or tuple(w_uk.shape) != ((heads * rank, dim) if transposed else (heads * dim, rank))
             or w_uk.dtype != out.dtype or tuple(cos.shape) != (n, rot_dim // 2) or tuple(sin.shape) != tuple(cos.shape)):
         raise KernelError("latent_query: shapes do not fit")
     F32 = torch.float32
     _launch("kllm_latent_query", "latent_query", _ptr(q, "latent q", F32), nsplit, stride, _ptr(w_uk, "latent w_uk"),
             _ptr(cos, "latent cos", F32), _ptr(sin, "latent sin", F32), _ptr(out, "latent q out"), n, int(heads),
-            int(dim), int(rot_dim), int(rank), dtype_code(out.dtype), _stream())
+            int(dim), int(rot_dim), int(rank), dtype_code(out.dtype), int(bool(transposed)), _stream())
 
 
-def attn_latent(q, out, cache, positions, span_of_token, block_table, page_size, heads, row, rank, scale, plain=False):
+def attn_latent_slices(n, heads, rank, dtype=torch.bfloat16) -> int:
+    """Workgroups that share out the keys of a token and 16 heads (their results are merged in
+    the same call): as many as bring a step's workgroups to about two a CU, for steps of few
+    tokens; 1 where the kernel on the matrix cores does not run.  Does not depend on any context
+    length, so a recorded step can be replayed as contexts grow."""
+    if dtype != torch.bfloat16 or rank % 16 or rank > 512:
+        return 1
+    groups = n * ((heads + 15) // 16)
+    slices = 1
+    while slices < 32 and groups * slices * 2 <= 2 * device_cus():
+        slices *= 2
+    return slices
+
+
+def attn_latent(q, out, cache, positions, span_of_token, block_table, page_size, heads, row, rank, scale, plain=False,
+                part=None, nslices=1):
     """Causal attention of q [n, H row] over cached rows of ``row`` elements whose first ``rank``
     are also the values (a page: its rows, then the first ``rank`` elements once more as
     [rank][slot]): out [n, H rank].  ``plain``: the kernel for every size, also where the one on
@@ -1762,7 +1779,8 @@ def attn_latent(q, out, cache, positions, span_of_token, block_table, page_size,
             _ptr(cache, "attn_latent cache"), _ptr(positions, "attn_latent positions", I32),
             _ptr(span_of_token, "attn_latent span_of_token", I32), _ptr(block_table, "attn_latent block_table", I32),
             block_table.shape[1], int(page_size), n, int(heads), int(row), int(rank), float(scale), dtype_code(q.dtype),
-            int(bool(plain)), _stream())
+            int(bool(plain)), _ptr(part, "attn_latent part", torch.float32, True) if nslices > 1 else 0,
+            part.numel() if nslices > 1 else 0, int(nslices), _stream())
 
 
 def latent_out(attended, w_uv, out, heads, vdim, rank, gate=None, gate_column=0):

@@ -79,12 +79,18 @@ class LatentAttention(Part):
         self.w_in = torch.cat(first, dim=0).contiguous()
         self.w_uq, self.w_uk, self.w_uv, self.w_o = w("uq.weight"), w("uk.weight"), w("uv.weight"), w("o.weight")
         self.q_norm, self.kv_norm = w("dq.norm"), w("dkv.norm")
+        # the matrix cores sum along a row: a second copy of W_uk, head by head [rank, head_dim]
+        self.w_ukt = None
+        if self.w_uk.dtype == torch.bfloat16 and self.head_dim % 32 == 0:
+            self.w_ukt = (self.w_uk.view(self.heads, self.head_dim, self.kv_rank).transpose(1, 2).contiguous()
+                          .view(self.heads * self.kv_rank, self.head_dim))
         self._tiled = {"in": tiled_copy(self.runtime, self.w_in, K.LINEAR_PARTS),
                        "uq": tiled_copy(self.runtime, self.w_uq, K.LINEAR_PARTS),
                        "o": tiled_copy(self.runtime, self.w_o, K.LINEAR_PARTS)}
 
     def tensors(self):
-        return [self.w_in, self.w_uq, self.w_uk, self.w_uv, self.w_o, self.q_norm, self.kv_norm]
+        return [self.w_in, self.w_uq, self.w_uk if self.w_ukt is None else self.w_ukt, self.w_uv, self.w_o, self.q_norm,
+                self.kv_norm]
 
     def cache_need(self):
         return CacheNeed("paged", kv_heads=1, head_dim=self.row, value_dim=self.kv_rank)
@@ -110,11 +116,16 @@ class LatentAttention(Part):
         K.latent_kv_append(first, self.q_rank, self.kv_norm, self.eps, cos, sin, cache.pages, ctx.positions,
                            ctx.span_of_token, cache.block_table, cache.page_size, self.kv_rank, self.rot_dim)
         qa = ctx.buf("latent.qa", (n, self.heads * self.row), dtype)
-        K.latent_query(q, self.w_uk, cos, sin, qa, self.heads, self.head_dim, self.rot_dim, self.kv_rank)
+        if self.w_ukt is not None:
+            K.latent_query(q, self.w_ukt, cos, sin, qa, self.heads, self.head_dim, self.rot_dim, self.kv_rank, transposed=True)
+        else:
+            K.latent_query(q, self.w_uk, cos, sin, qa, self.heads, self.head_dim, self.rot_dim, self.kv_rank)
         attended = ctx.buf("latent.att", (n, self.heads * self.kv_rank), dtype)
+        plain = self.runtime.options.get("attention", "auto") == "generic"
+        slices = 1 if plain or self.row % 8 or cache.page_size % 16 else K.attn_latent_slices(n, self.heads, self.kv_rank, dtype)
+        part = ctx.buf("latent.part", (n * self.heads * slices * (self.kv_rank + 2),), torch.float32) if slices > 1 else None
         K.attn_latent(qa, attended, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table, cache.page_size,
-                      self.heads, self.row, self.kv_rank, self.scale,
-                      plain=self.runtime.options.get("attention", "auto") == "generic")
+                      self.heads, self.row, self.kv_rank, self.scale, plain=plain, part=part, nslices=slices)
         out = ctx.buf("latent.out", (n, self.out_dim), dtype)
         K.latent_out(attended, self.w_uv, out, self.heads, self.value_dim, self.kv_rank,
                      gate=first if self.gated else None, gate_column=self.q_rank + self.row)

@@ -306,14 +306,54 @@ def test_attention_over_cached_latents(H, rank, dr, dtype):
         base += nl
     assert float(torch.softmax(torch.einsum("hd,kd->hk", qq[400], stored[:401]) * scale, -1)[:, 3].min()) > 0.5
     tol = 2e-5 if dtype == "float32" else 1.5e-2
-    for plain in (True, False):
+    for plain, slices in ((True, 1), (False, 1), (False, 4), (False, 32)):
         out = torch.zeros(n, H * rank, device="cuda", dtype=dt)
-        K.attn_latent(qd, out, cache, i32(positions), i32(span_of), table.cuda(), page, H, row, rank, scale, plain=plain)
+        part = torch.full((n * H * slices * (rank + 2),), float("nan"), device="cuda") if slices > 1 else None
+        K.attn_latent(qd, out, cache, i32(positions), i32(span_of), table.cuda(), page, H, row, rank, scale, plain=plain,
+                      part=part, nslices=slices)
         got = out.float().cpu().reshape(n, H, rank)
         assert torch.isfinite(got).all()
         for i in (0, 1, 15, 16, 17, 400, 430, 431, 449):
-            assert rel(got[i], want[i]) < tol, (plain, i)
-        assert rel(got, want) < tol, plain
+            assert rel(got[i], want[i]) < tol, (plain, slices, i)
+        assert rel(got, want) < tol, (plain, slices)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,H,d,dr,dv,rank", [(1, 3, 16, 8, 20, 40), (37, 6, 64, 32, 64, 160), (130, 3, 128, 64, 128, 448),
+                                              (5, 20, 32, 16, 24, 96), (70, 2, 96, 8, 200, 64)])
+def test_the_products_with_a_heads_own_matrices(n, H, d, dr, dv, rank, dtype):
+    """The query folded through W_uk (as stored, and head by head transposed for the matrix cores)
+    with its rotated part, and the attended latent through W_uv times the gate."""
+    from kllm_amd import kernels as K
+    dt = {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype]
+    g = torch.Generator().manual_seed(n + rank)
+    tol = 2e-6 if dtype == "float32" else 8e-3
+    qs = torch.randn(2, n, H * (d + dr), generator=g)
+    w_uk = (torch.randn(H * d, rank, generator=g) / d ** 0.5).to(dt)
+    positions = [3 * i + 1 for i in range(n)]
+    rot = {"dims": dr, "base": 900.0}
+    cos, sin = torch.empty(n, dr // 2, device="cuda"), torch.empty(n, dr // 2, device="cuda")
+    K.rope_tables_freq(cos, sin, torch.tensor(positions, dtype=torch.int32, device="cuda"), P.frequencies(rot).cuda(), 1.0)
+    q = qs.double().sum(0).reshape(n, H, d + dr)
+    want = torch.cat([torch.einsum("nhi,hir->nhr", q[..., :d], w_uk.double().reshape(H, d, rank)),
+                      P.rotate_halves(q[..., d:], positions, rot)], dim=-1).reshape(n, H * (rank + dr))
+    out = torch.empty(n, H * (rank + dr), device="cuda", dtype=dt)
+    K.latent_query(qs.cuda(), w_uk.cuda(), cos, sin, out, H, d, dr, rank)
+    assert rel(out.float().cpu(), want) < tol
+    if dtype == "bfloat16" and d % 32 == 0:
+        w_t = w_uk.reshape(H, d, rank).transpose(1, 2).contiguous().reshape(H * rank, d)
+        out.fill_(float("nan"))
+        K.latent_query(qs.cuda(), w_t.cuda(), cos, sin, out, H, d, dr, rank, transposed=True)
+        assert rel(out.float().cpu(), want) < tol
+    att = torch.randn(n, H * rank, generator=g).to(dt)
+    w_uv = (torch.randn(H * dv, rank, generator=g) / rank ** 0.5).to(dt)
+    gate = torch.randn(3, n, 7 + H * dv, generator=g)
+    want = torch.einsum("nhr,hjr->nhj", att.double().reshape(n, H, rank), w_uv.double().reshape(H, dv, rank)).reshape(n, H * dv)
+    out = torch.full((n, H * dv), float("nan"), device="cuda", dtype=dt)
+    K.latent_out(att.cuda(), w_uv.cuda(), out, H, dv, rank)
+    assert rel(out.float().cpu(), want) < tol
+    K.latent_out(att.cuda(), w_uv.cuda(), out, H, dv, rank, gate=gate.cuda(), gate_column=7)
+    assert rel(out.float().cpu(), want * torch.sigmoid(gate.double().sum(0)[:, 7:])) < tol
 
 
 # ----------------------------------------------------------------------------- each mixer alone
