@@ -278,27 +278,62 @@ __global__ __launch_bounds__(kRecThreads) void linear_recurrence_prep_kernel(
   }
 }
 
-// S <- a S + b along a span, one thread a (span, channel); out = S * gelu_tanh(y + y_bias).  Eight
-// tokens' numbers are asked for at a time, so that the chain holds arithmetic only.
+// S <- a S + b along a span; out = S * gelu_tanh(y + y_bias).  Eight tokens' numbers are asked
+// for at a time, so that the chain holds arithmetic only.
+// A span's tokens are cut into kScanSegs segments, one wave each (64 channels a workgroup):
+// S_t = a_t S_(t-1) + b_t is a composition of maps S -> a S + b, and so is a whole segment's
+// (A S + B, with A the product of its a and B its own chain from zero).  Every wave first runs its
+// segment's chain from zero, the segments' (A, B) meet in LDS, a wave folds those before its own
+// into its starting state and runs its segment once more, now writing.  A chain of n steps
+// becomes two of n / kScanSegs.
+constexpr int kScanCh = 64;
+constexpr int kScanSegs = 16;
+
 template <typename T>
-__global__ __launch_bounds__(kRecThreads) void linear_recurrence_scan_kernel(
+__global__ __launch_bounds__(kScanCh * kScanSegs) void linear_recurrence_scan_kernel(
     const float* __restrict__ a_in, const float* __restrict__ b_in, const float* __restrict__ proj, int nsplit,
     long split_stride, const float* __restrict__ y_bias, float* __restrict__ state, long slot_stride,
     const int* __restrict__ slots, const int* __restrict__ span_start, const int* __restrict__ span_pos,
     T* __restrict__ out, int W) {
-  const int c = blockIdx.x * kRecThreads + threadIdx.x;
-  if (c >= W) return;
+  __shared__ float seg_a[kScanSegs][kScanCh], seg_b[kScanSegs][kScanCh];
+  const int lane = threadIdx.x % kScanCh, seg = threadIdx.x / kScanCh;
+  const int c = min((int)blockIdx.x * kScanCh + lane, W - 1);
+  const bool ok = blockIdx.x * kScanCh + lane < W;
   const int span = blockIdx.y;
   const long t0 = span_start[span], t1 = span_start[span + 1];
+  const long per = (t1 - t0 + kScanSegs - 1) / kScanSegs;
+  const long a0 = min(t1, t0 + seg * per), a1 = min(t1, a0 + per);
+  constexpr int U = 8;
+  float A = 1.f, B = 0.f;
+  {
+    for (long tb = a0; tb < a1; tb += U) {
+      float a[U], b[U];
+#pragma unroll
+      for (int q = 0; q < U; ++q) {
+        const long t = min(tb + q, a1 - 1);
+        a[q] = a_in[t * W + c];
+        b[q] = b_in[t * W + c];
+      }
+#pragma unroll
+      for (int q = 0; q < U; ++q) {
+        if (tb + q >= a1) break;
+        B = fmaf(a[q], B, b[q]);
+        A *= a[q];
+      }
+    }
+  }
+  seg_a[seg][lane] = A;
+  seg_b[seg][lane] = B;
+  __syncthreads();
   float* st = state + (long)slots[span] * slot_stride + c;
   float S = span_pos[span] == 0 ? 0.f : *st;
+  for (int s = 0; s < seg; ++s) S = fmaf(seg_a[s][lane], S, seg_b[s][lane]);
   const float yb = y_bias[c];
-  constexpr int U = 8;
-  for (long tb = t0; tb < t1; tb += U) {
+  for (long tb = a0; tb < a1; tb += U) {
     float a[U], b[U], y[U];
 #pragma unroll
     for (int q = 0; q < U; ++q) {
-      const long t = min(tb + q, t1 - 1);
+      const long t = min(tb + q, a1 - 1);
       a[q] = a_in[t * W + c];
       b[q] = b_in[t * W + c];
       float v = 0.f;
@@ -307,12 +342,13 @@ __global__ __launch_bounds__(kRecThreads) void linear_recurrence_scan_kernel(
     }
 #pragma unroll
     for (int q = 0; q < U; ++q) {
-      if (tb + q >= t1) break;
+      if (tb + q >= a1) break;
       S = fmaf(a[q], S, b[q]);
-      out[(tb + q) * W + c] = from_f32<T>(S * y[q]);
+      if (ok) out[(tb + q) * W + c] = from_f32<T>(S * y[q]);
     }
   }
-  *st = S;
+  // the wave of the last segment ends at the span's last token (an empty segment has folded all)
+  if (ok && seg == kScanSegs - 1) *st = S;
 }
 
 // out = sa * (sum of a's slices) + sb * (sum of b's slices), element by element.
@@ -431,12 +467,12 @@ extern "C" int kllm_linear_recurrence_scan(const float* a_in, const float* b_in,
   KLLM_REQUIRE(n_spans > 0 && n_spans <= 65535 && W > 0 && nsplit >= 1, "linear_recurrence_scan: bad sizes spans=%d W=%d",
                n_spans, W);
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "linear_recurrence_scan: unknown dtype %d", dtype);
-  const dim3 grid(ceil_div(W, kRecThreads), n_spans);
+  const dim3 grid(ceil_div(W, kScanCh), n_spans);
   if (dtype == DT_F32)
-    hipLaunchKernelGGL(linear_recurrence_scan_kernel<float>, grid, dim3(kRecThreads), 0, stream, a_in, b_in, proj,
+    hipLaunchKernelGGL(linear_recurrence_scan_kernel<float>, grid, dim3(kScanCh * kScanSegs), 0, stream, a_in, b_in, proj,
                        nsplit, split_stride, y_bias, state, slot_stride, slots, span_start, span_pos, (float*)out, W);
   else
-    hipLaunchKernelGGL(linear_recurrence_scan_kernel<bf16_t>, grid, dim3(kRecThreads), 0, stream, a_in, b_in, proj,
+    hipLaunchKernelGGL(linear_recurrence_scan_kernel<bf16_t>, grid, dim3(kScanCh * kScanSegs), 0, stream, a_in, b_in, proj,
                        nsplit, split_stride, y_bias, state, slot_stride, slots, span_start, span_pos, (bf16_t*)out, W);
   KLLM_CHECK_LAUNCH("linear_recurrence_scan");
   return 0;
