@@ -163,4 +163,25 @@ int device_xcds();
 
 inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }
 
+// Sum over the PARTS neighbouring lanes that share a column (PARTS a power of two up to 64), every
+// lane getting the sum: within a row of 16 lanes by data-parallel moves (neighbour, other pair,
+// mirrored half row, mirrored row), which cost an instruction each; across the two rows of a
+// group of 32 by a lane exchange.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true);   // (every lane has a source: the move folds into the add)
+  return v + __builtin_bit_cast(float, moved);
+}
+
+template <int PARTS>
+__device__ __forceinline__ float parts_sum(float v) {
+  if (PARTS >= 2) v = dpp_add<0xB1>(v);     // quad_perm [1,0,3,2]
+  if (PARTS >= 4) v = dpp_add<0x4E>(v);     // quad_perm [2,3,0,1]
+  if (PARTS >= 8) v = dpp_add<0x141>(v);    // row_half_mirror
+  if (PARTS >= 16) v = dpp_add<0x140>(v);   // row_mirror
+  if (PARTS >= 32) v += __shfl_xor(v, 16, kWave);
+  if (PARTS >= 64) v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+
 }  // namespace kllm

@@ -211,7 +211,9 @@ __global__ __launch_bounds__(kLatThreads) void attn_latent_kernel(
 // 8-byte reads from the transposed copy.  NR: 16-element pieces of the latent a lane accumulates.
 constexpr int kLatWaves = 4;
 
-template <int NR>
+// KS: steps of 32 over a row whose pieces of the query a lane keeps in registers (0: it asks for
+// them at every tile, for rows longer than the built sizes).
+template <int NR, int KS>
 __global__ __launch_bounds__(64 * kLatWaves) void attn_latent_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ span_of_token, const int* __restrict__ block_table,
@@ -228,6 +230,12 @@ __global__ __launch_bounds__(64 * kLatWaves) void attn_latent_mfma_kernel(
   const int ksteps = (row + 31) / 32, nr = rank / 16;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   const bf16_t* qrow = q + ((long)t * H + head) * row;
+  bf16x8 qreg[KS > 0 ? KS : 1];
+#pragma unroll
+  for (int kk = 0; kk < KS; ++kk) {
+    const int d0 = 32 * kk + 8 * g;
+    qreg[kk] = (d0 < row && head_ok) ? *reinterpret_cast<const bf16x8*>(qrow + d0) : zero8;
+  }
 
   float m = -INFINITY, l = 0.f;
   floatx4 acc[NR];
@@ -253,14 +261,23 @@ __global__ __launch_bounds__(64 * kLatWaves) void attn_latent_mfma_kernel(
       slot0[u] = live[u] ? k0 % page_size : 0;
     }
     floatx4 s[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
-    for (int ks = 0; ks < ksteps; ++ks) {
+    auto score_step = [&](int ks, const bf16x8& qb) {
       const int d0 = 32 * ks + 8 * g;
       const bool in = d0 < row;
-      const bf16x8 qb = (in && head_ok) ? *reinterpret_cast<const bf16x8*>(qrow + d0) : zero8;
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         const bf16x8 a = (in && live[u]) ? *reinterpret_cast<const bf16x8*>(pbase[u] + (long)(slot0[u] + c) * row + d0) : zero8;
         s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb, s[u], 0, 0, 0);
+      }
+    };
+    if constexpr (KS > 0) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        if (ks < ksteps) score_step(ks, qreg[ks]);
+    } else {
+      for (int ks = 0; ks < ksteps; ++ks) {
+        const int d0 = 32 * ks + 8 * g;
+        score_step(ks, (d0 < row && head_ok) ? *reinterpret_cast<const bf16x8*>(qrow + d0) : zero8);
       }
     }
     // ---- online softmax for this lane's head over its 8 keys, then over the 4 lanes of the column
@@ -378,6 +395,165 @@ __global__ __launch_bounds__(64 * kLatWaves) void attn_latent_mfma_kernel(
   }
 }
 
+// The same for steps of many tokens: a workgroup takes four consecutive tokens of the step and up
+// to 16 heads, one token a wave.  Tokens of one request read the same keys: a tile of 32 keys
+// (their rows, and their latents with the keys side by side) goes through LDS once for the
+// four, which cuts the traffic between L2 and the CUs to a quarter.  Where the four tokens
+// belong to several requests, the requests take their turns.  No merge: a wave has all keys
+// of its token.  LDS: rows [32][row + 8], latents [rank][32 + 4] (padded against bank conflicts).
+template <int NR, int KS>
+__global__ __launch_bounds__(64 * kLatWaves) void attn_latent_block_kernel(
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
+    const int* __restrict__ positions, const int* __restrict__ span_of_token, const int* __restrict__ block_table,
+    int max_pages, int page_size, int n, int H, int row, int rank, float scale) {
+  extern __shared__ __attribute__((aligned(16))) bf16_t lat_tiles[];
+  const int KLD = row + 8, VLD = 36;
+  bf16_t* ks = lat_tiles;                      // [32][KLD]
+  bf16_t* vs = lat_tiles + 32 * KLD;           // [rank][VLD]
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int g = lane / 16, c = lane % 16;
+  const int t_first = blockIdx.x * kLatWaves, h0 = blockIdx.y * 16;
+  const int t = min(t_first + wave, n - 1);
+  const bool token_ok = t_first + wave < n;
+  const int head = min(h0 + c, H - 1);
+  const bool head_ok = h0 + c < H;
+  const int my_span = span_of_token[t];
+  const int len = positions[t] + 1;
+  const long page_elems = (long)page_size * (row + rank);
+  const int ksteps = (row + 31) / 32, nr = rank / 16;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const bf16_t* qrow = q + ((long)t * H + head) * row;
+  const int rows_here = min(kLatWaves, n - t_first);
+  bf16x8 qreg[KS > 0 ? KS : 1];
+#pragma unroll
+  for (int kk = 0; kk < KS; ++kk) {
+    const int d0 = 32 * kk + 8 * g;
+    qreg[kk] = (d0 < row && head_ok) ? *reinterpret_cast<const bf16x8*>(qrow + d0) : zero8;
+  }
+
+  float m = -INFINITY, l = 0.f;
+  floatx4 acc[NR];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) acc[r] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  for (int first = 0; first < rows_here;) {
+    const int span = span_of_token[t_first + first];
+    int last = first;
+    while (last + 1 < rows_here && span_of_token[t_first + last + 1] == span) ++last;
+    const int group_len = positions[t_first + last] + 1;      // the group's last token reads the most keys
+    const bool mine = token_ok && wave >= first && wave <= last;
+    const int* table = block_table + (long)span * max_pages;
+    for (int kb = 0; kb < group_len; kb += 32) {
+      __syncthreads();                                        // the tile before this one has been read
+      // ---- the tile's way into LDS: 16-byte pieces; a half (16 keys) lies in one page
+      const int row8 = row / 8;
+      for (int i = tid; i < 32 * row8; i += 64 * kLatWaves) {
+        const int kr = i / row8, piece = i % row8;
+        const int key = kb + kr;
+        bf16x8 v = zero8;
+        if (key < group_len) {
+          const long pg = table[key / page_size];
+          v = *reinterpret_cast<const bf16x8*>(cache + pg * page_elems + (long)(key % page_size) * row + 8 * piece);
+        }
+        *reinterpret_cast<bf16x8*>(ks + kr * KLD + 8 * piece) = v;
+      }
+      for (int i = tid; i < rank * 4; i += 64 * kLatWaves) {
+        const int e = i / 4, part = i % 4;                    // 8 keys of one element
+        const int key = kb + 8 * part;
+        bf16x8 v = zero8;
+        if (key < group_len) {
+          const long pg = table[key / page_size];
+          v = *reinterpret_cast<const bf16x8*>(cache + pg * page_elems + (long)page_size * row + (long)e * page_size +
+                                               key % page_size);
+          if (key + 8 > group_len) {                          // slots behind the last key may hold anything
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = key + j < group_len ? v[j] : (bf16_t)0.f;
+          }
+        }
+        bf16_t* dst = vs + e * VLD + 8 * part;                // 8-byte aligned
+        *reinterpret_cast<bf16x4*>(dst) = bf16x4{v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<bf16x4*>(dst + 4) = bf16x4{v[4], v[5], v[6], v[7]};
+      }
+      __syncthreads();
+      if (!mine || kb >= len) continue;
+      // ---- scores
+      floatx4 s[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
+      auto score_step = [&](int kk, const bf16x8& qb) {
+        const int d0 = 32 * kk + 8 * g;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const bf16x8 a = d0 < row ? *reinterpret_cast<const bf16x8*>(ks + (16 * u + c) * KLD + d0) : zero8;
+          s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb, s[u], 0, 0, 0);
+        }
+      };
+      if constexpr (KS > 0) {
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk)
+          if (kk < ksteps) score_step(kk, qreg[kk]);
+      } else {
+        for (int kk = 0; kk < ksteps; ++kk) {
+          const int d0 = 32 * kk + 8 * g;
+          score_step(kk, (d0 < row && head_ok) ? *reinterpret_cast<const bf16x8*>(qrow + d0) : zero8);
+        }
+      }
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kb + 16 * u + 4 * g + i;
+          s[u][i] = key < len ? s[u][i] * scale : -INFINITY;
+          tmax = fmaxf(tmax, s[u][i]);
+        }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+      const float m_new = fmaxf(m, tmax);                    // finite: kb < len
+      const float alpha = expf(m - m_new);
+      bf16x8 pb;
+      float psum = 0.f;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = (s[u][i] == -INFINITY) ? 0.f : expf(s[u][i] - m_new);
+          const bf16_t pr = (bf16_t)p;
+          pb[4 * u + i] = pr;
+          psum += (float)pr;
+        }
+      l = l * alpha + psum;
+      m = m_new;
+      // ---- the weighted sum of the latents (keys beyond this token's last: probability 0, and
+      // what LDS holds of them is another token's key or zero, never anything else)
+#pragma unroll
+      for (int r = 0; r < NR; ++r) {
+        if (r < nr) {
+          acc[r] *= alpha;
+          const bf16_t* vrow = vs + (16 * r + c) * VLD + 4 * g;
+          const bf16x4 lo = *reinterpret_cast<const bf16x4*>(vrow);
+          const bf16x4 hi = *reinterpret_cast<const bf16x4*>(vrow + 16);
+          const bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[r], 0, 0, 0);
+        }
+      }
+    }
+    first = last + 1;
+  }
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+  if (!token_ok || !head_ok) return;
+  const float inv = 1.f / l;
+  bf16_t* orow = out + ((long)t * H + head) * rank;
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    if (r < nr) {
+      bf16x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = (bf16_t)(acc[r][i] * inv);
+      *reinterpret_cast<bf16x4*>(orow + 16 * r + 4 * g) = v;
+    }
+  }
+}
+
 // The slices' results of one (token, head) become its output: weights exp(m_s - max m).
 __global__ __launch_bounds__(kLatThreads) void attn_latent_merge_kernel(const float* __restrict__ part,
                                                                         bf16_t* __restrict__ out, int rank, int nslices) {
@@ -401,17 +577,29 @@ __global__ __launch_bounds__(kLatThreads) void attn_latent_merge_kernel(const fl
   }
 }
 
-template <int NR>
+template <int NR, int KS>
 static void launch_latent_mfma(const void* q, void* out, const void* cache, const int* positions, const int* span_of_token,
                                const int* block_table, int max_pages, int page_size, int n, int H, int row, int rank,
                                float scale, float* part, int nslices, hipStream_t stream) {
   const size_t lds = (size_t)(kLatWaves - 1) * (NR * 4 + 2) * kWave * sizeof(float);
   static int raised = 0;
   if (lds > 64 * 1024 && !raised) {
-    (void)hipFuncSetAttribute((const void*)attn_latent_mfma_kernel<NR>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    (void)hipFuncSetAttribute((const void*)attn_latent_mfma_kernel<NR, KS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     raised = 1;
   }
-  hipLaunchKernelGGL(attn_latent_mfma_kernel<NR>, dim3(n, (H + 15) / 16, nslices), dim3(64 * kLatWaves), lds, stream,
+  if (nslices == 0) {       // steps of many tokens: four tokens a workgroup, their keys through LDS
+    const size_t tiles = ((size_t)32 * (row + 8) + (size_t)rank * 36) * sizeof(bf16_t);
+    static size_t raised_to = 64 * 1024;
+    if (tiles > raised_to) {
+      (void)hipFuncSetAttribute((const void*)attn_latent_block_kernel<NR, KS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)tiles);
+      raised_to = tiles;
+    }
+    hipLaunchKernelGGL((attn_latent_block_kernel<NR, KS>), dim3((n + kLatWaves - 1) / kLatWaves, (H + 15) / 16), dim3(64 * kLatWaves),
+                       tiles, stream, (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, positions, span_of_token,
+                       block_table, max_pages, page_size, n, H, row, rank, scale);
+    return;
+  }
+  hipLaunchKernelGGL((attn_latent_mfma_kernel<NR, KS>), dim3(n, (H + 15) / 16, nslices), dim3(64 * kLatWaves), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, positions, span_of_token, block_table, max_pages,
                      page_size, H, row, rank, scale, part);
   if (nslices > 1)
@@ -614,12 +802,16 @@ extern "C" int kllm_attn_latent(const void* q, void* out, const void* cache, con
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "attn_latent: unknown dtype %d", dtype);
   if (dtype == DT_BF16 && mode != 1 && rank % 16 == 0 && row % 8 == 0 && rank <= 512 && page_size % 16 == 0 &&
       ((uintptr_t)q & 15) == 0 && ((uintptr_t)cache & 15) == 0 && ((uintptr_t)out & 7) == 0) {
-    KLLM_REQUIRE(nslices >= 1 && nslices <= 64 && (nslices == 1 || (part && part_floats >= (long)n * H * nslices * (rank + 2))),
+    KLLM_REQUIRE(nslices >= 0 && nslices <= 64 && (nslices <= 1 || (part && part_floats >= (long)n * H * nslices * (rank + 2))),
                  "attn_latent: %d slices need room for %d tokens x %d heads x %d slices x (%d + 2) floats", nslices, n, H,
                  nslices, rank);
-    if (rank <= 128) launch_latent_mfma<8>(q, out, cache, positions, span_of_token, block_table, max_pages, page_size, n, H, row, rank, scale, part, nslices, stream);
-    else if (rank <= 256) launch_latent_mfma<16>(q, out, cache, positions, span_of_token, block_table, max_pages, page_size, n, H, row, rank, scale, part, nslices, stream);
-    else launch_latent_mfma<32>(q, out, cache, positions, span_of_token, block_table, max_pages, page_size, n, H, row, rank, scale, part, nslices, stream);
+    // the latent's accumulators and the query's pieces in registers: built for ranks up to 128, 256 and
+    // 512 with rows of up to 256, 384 and 640; longer rows ask for the query at every tile
+#define KLLM_LAT(NR, KS) launch_latent_mfma<NR, KS>(q, out, cache, positions, span_of_token, block_table, max_pages, page_size, n, H, row, rank, scale, part, nslices, stream)
+    if (rank <= 128) { if (row <= 256) KLLM_LAT(8, 8); else KLLM_LAT(8, 0); }
+    else if (rank <= 256) { if (row <= 384) KLLM_LAT(16, 12); else KLLM_LAT(16, 0); }
+    else { if (row <= 640) KLLM_LAT(32, 20); else KLLM_LAT(32, 0); }
+#undef KLLM_LAT
     KLLM_CHECK_LAUNCH("attn_latent");
     return 0;
   }

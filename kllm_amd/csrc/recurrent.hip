@@ -195,8 +195,7 @@ __global__ __launch_bounds__(kRecThreads) void gated_delta_scan_kernel(
         s[i] *= decay;
         dot = fmaf(s[i], kr[i], dot);
       }
-#pragma unroll
-      for (int off = 1; off < kDeltaParts; off <<= 1) dot += __shfl_xor(dot, off, kWave);
+      dot = parts_sum<kDeltaParts>(dot);
       const float u = beta * (vs[tt * kDeltaCols + jl] - dot);
       float o = 0.f;
 #pragma unroll
@@ -205,8 +204,7 @@ __global__ __launch_bounds__(kRecThreads) void gated_delta_scan_kernel(
         s[i] = fmaf(kr[i], u, s[i]);
         o = fmaf(s[i], r < dk ? qt[r] : 0.f, o);
       }
-#pragma unroll
-      for (int off = 1; off < kDeltaParts; off <<= 1) o += __shfl_xor(o, off, kWave);
+      o = parts_sum<kDeltaParts>(o);
       if (col && p == 0) o_out[(tb + tt) * HV + (long)h * dv + j] = o;
     }
   }

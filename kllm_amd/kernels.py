@@ -1749,13 +1749,19 @@ def latent_query(q, w_uk, cos, sin, out, heads, dim, rot_dim, rank, transposed=F
             int(dim), int(rot_dim), int(rank), dtype_code(out.dtype), int(bool(transposed)), _stream())
 
 
+LATENT_BLOCK_FROM = 64      # tokens of a step from which four tokens share a workgroup and its tiles of keys
+
+
 def attn_latent_slices(n, heads, rank, dtype=torch.bfloat16) -> int:
     """Workgroups that share out the keys of a token and 16 heads (their results are merged in
     the same call): as many as bring a step's workgroups to about two a CU, for steps of few
-    tokens; 1 where the kernel on the matrix cores does not run.  Does not depend on any context
+    tokens; 1 where the kernel on the matrix cores does not run; 0 for steps of many tokens: there
+    a workgroup takes four tokens, whose keys pass through LDS once for the four.  Does not depend on any context
     length, so a recorded step can be replayed as contexts grow."""
     if dtype != torch.bfloat16 or rank % 16 or rank > 512:
         return 1
+    if n >= LATENT_BLOCK_FROM:
+        return 0
     groups = n * ((heads + 15) // 16)
     slices = 1
     while slices < 32 and groups * slices * 2 <= 2 * device_cus():

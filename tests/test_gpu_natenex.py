@@ -306,7 +306,7 @@ def test_attention_over_cached_latents(H, rank, dr, dtype):
         base += nl
     assert float(torch.softmax(torch.einsum("hd,kd->hk", qq[400], stored[:401]) * scale, -1)[:, 3].min()) > 0.5
     tol = 2e-5 if dtype == "float32" else 1.5e-2
-    for plain, slices in ((True, 1), (False, 1), (False, 4), (False, 32)):
+    for plain, slices in ((True, 1), (False, 1), (False, 4), (False, 32), (False, 0)):    # 0: four tokens a workgroup
         out = torch.zeros(n, H * rank, device="cuda", dtype=dt)
         part = torch.full((n * H * slices * (rank + 2),), float("nan"), device="cuda") if slices > 1 else None
         K.attn_latent(qd, out, cache, i32(positions), i32(span_of), table.cuda(), page, H, row, rank, scale, plain=plain,
