@@ -217,7 +217,7 @@ template <int NR, int KS>
 __global__ __launch_bounds__(64 * kLatWaves) void attn_latent_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ span_of_token, const int* __restrict__ block_table,
-    int max_pages, int page_size, int H, int row, int rank, float scale, float* __restrict__ part) {
+    int max_pages, int page_size, unsigned page_magic, int H, int row, int rank, float scale, float* __restrict__ part) {
   extern __shared__ float lat_red[];            // [kLatWaves - 1][NR * 4 + 2][64]
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int g = lane / 16, c = lane % 16;
@@ -256,9 +256,10 @@ __global__ __launch_bounds__(64 * kLatWaves) void attn_latent_mfma_kernel(
     for (int u = 0; u < 2; ++u) {
       const int k0 = kb + 16 * u;
       live[u] = k0 < len;
-      const int page = table[live[u] ? k0 / page_size : 0];
+      const int pi = live[u] ? (int)(__umulhi((unsigned)k0, page_magic) >> 3) : 0;   // k0 / page_size (see the launch)
+      const int page = table[pi];
       pbase[u] = cache + (long)page * page_elems;
-      slot0[u] = live[u] ? k0 % page_size : 0;
+      slot0[u] = live[u] ? k0 - pi * page_size : 0;
     }
     floatx4 s[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
     auto score_step = [&](int ks, const bf16x8& qb) {
@@ -405,14 +406,18 @@ template <int NR, int KS>
 __global__ __launch_bounds__(64 * kLatWaves) void attn_latent_block_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ span_of_token, const int* __restrict__ block_table,
-    int max_pages, int page_size, int n, int H, int row, int rank, float scale) {
+    int max_pages, int page_size, unsigned page_magic, int n, int H, int row, int rank, float scale) {
   extern __shared__ __attribute__((aligned(16))) bf16_t lat_tiles[];
+  // page of a key without a division: page_magic = ceil(2^35 / page_size) from the host, exact for
+  // keys below 2^24 and pages of up to 2,048 slots (checked at the launch)
+  auto page_index = [&](int key) { return (int)(__umulhi((unsigned)key, page_magic) >> 3); };
   const int KLD = row + 8, VLD = 36;
   bf16_t* ks = lat_tiles;                      // [32][KLD]
   bf16_t* vs = lat_tiles + 32 * KLD;           // [rank][VLD]
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int g = lane / 16, c = lane % 16;
-  const int t_first = blockIdx.x * kLatWaves, h0 = blockIdx.y * 16;
+  // later tokens of a prompt read more keys: the workgroups with the most to do start first
+  const int t_first = (gridDim.x - 1 - blockIdx.x) * kLatWaves, h0 = blockIdx.y * 16;
   const int t = min(t_first + wave, n - 1);
   const bool token_ok = t_first + wave < n;
   const int head = min(h0 + c, H - 1);
@@ -443,38 +448,70 @@ __global__ __launch_bounds__(64 * kLatWaves) void attn_latent_block_kernel(
     const int group_len = positions[t_first + last] + 1;      // the group's last token reads the most keys
     const bool mine = token_ok && wave >= first && wave <= last;
     const int* table = block_table + (long)span * max_pages;
+    // ---- a tile's way into LDS: 16-byte pieces (a half, 16 keys, lies in one page).  For the built
+    // row sizes a thread's pieces of the NEXT tile are asked for before the products of this one
+    // and wait in registers meanwhile.
+    const int row8 = row / 8;
+    constexpr int KP = KS / 2, VP = NR / 4;     // pieces a thread: 32 rows x 4 KS / 256, 16 NR elements x 4 / 256
+    struct Stage {
+      bf16x8 k[KP > 0 ? KP : 1], v[VP];
+    };
+    auto k_piece = [&](int i, int kb) -> bf16x8 {
+      const int kr = i / row8;                                // (for the built sizes: unrolled, i and row8 known per thread before the loop)
+      const int key = kb + kr;
+      if (i >= 32 * row8 || key >= group_len) return zero8;
+      const int pi = page_index(key);
+      const long pg = table[pi];
+      return *reinterpret_cast<const bf16x8*>(cache + pg * page_elems + (long)(key - pi * page_size) * row + 8 * (i - kr * row8));
+    };
+    auto v_piece = [&](int i, int kb) -> bf16x8 {             // 8 keys of one element
+      const int e = i / 4, key = kb + 8 * (i % 4);
+      if (e >= rank || key >= group_len) return zero8;
+      const int pi = page_index(key);
+      const long pg = table[pi];
+      bf16x8 v = *reinterpret_cast<const bf16x8*>(cache + pg * page_elems + (long)page_size * row + (long)e * page_size +
+                                                  (key - pi * page_size));
+      if (key + 8 > group_len) {                              // slots behind the last key may hold anything
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = key + j < group_len ? v[j] : (bf16_t)0.f;
+      }
+      return v;
+    };
+    auto k_store = [&](int i, const bf16x8& v) {
+      const int kr = i / row8;
+      if (i < 32 * row8) *reinterpret_cast<bf16x8*>(ks + kr * KLD + 8 * (i - kr * row8)) = v;
+    };
+    auto v_store = [&](int i, const bf16x8& v) {
+      if (i >= rank * 4) return;
+      bf16_t* dst = vs + (i / 4) * VLD + 8 * (i % 4);         // 8-byte aligned
+      *reinterpret_cast<bf16x4*>(dst) = bf16x4{v[0], v[1], v[2], v[3]};
+      *reinterpret_cast<bf16x4*>(dst + 4) = bf16x4{v[4], v[5], v[6], v[7]};
+    };
+    auto fetch = [&](int kb) -> Stage {
+      Stage T;
+#pragma unroll
+      for (int j = 0; j < KP; ++j) T.k[j] = k_piece(tid + 64 * kLatWaves * j, kb);
+#pragma unroll
+      for (int j = 0; j < VP; ++j) T.v[j] = v_piece(tid + 64 * kLatWaves * j, kb);
+      return T;
+    };
+    Stage st;
+    if constexpr (KS > 0) st = fetch(0);
     for (int kb = 0; kb < group_len; kb += 32) {
       __syncthreads();                                        // the tile before this one has been read
-      // ---- the tile's way into LDS: 16-byte pieces; a half (16 keys) lies in one page
-      const int row8 = row / 8;
-      for (int i = tid; i < 32 * row8; i += 64 * kLatWaves) {
-        const int kr = i / row8, piece = i % row8;
-        const int key = kb + kr;
-        bf16x8 v = zero8;
-        if (key < group_len) {
-          const long pg = table[key / page_size];
-          v = *reinterpret_cast<const bf16x8*>(cache + pg * page_elems + (long)(key % page_size) * row + 8 * piece);
-        }
-        *reinterpret_cast<bf16x8*>(ks + kr * KLD + 8 * piece) = v;
-      }
-      for (int i = tid; i < rank * 4; i += 64 * kLatWaves) {
-        const int e = i / 4, part = i % 4;                    // 8 keys of one element
-        const int key = kb + 8 * part;
-        bf16x8 v = zero8;
-        if (key < group_len) {
-          const long pg = table[key / page_size];
-          v = *reinterpret_cast<const bf16x8*>(cache + pg * page_elems + (long)page_size * row + (long)e * page_size +
-                                               key % page_size);
-          if (key + 8 > group_len) {                          // slots behind the last key may hold anything
+      if constexpr (KS > 0) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] = key + j < group_len ? v[j] : (bf16_t)0.f;
-          }
-        }
-        bf16_t* dst = vs + e * VLD + 8 * part;                // 8-byte aligned
-        *reinterpret_cast<bf16x4*>(dst) = bf16x4{v[0], v[1], v[2], v[3]};
-        *reinterpret_cast<bf16x4*>(dst + 4) = bf16x4{v[4], v[5], v[6], v[7]};
+        for (int j = 0; j < KP; ++j) k_store(tid + 64 * kLatWaves * j, st.k[j]);
+#pragma unroll
+        for (int j = 0; j < VP; ++j) v_store(tid + 64 * kLatWaves * j, st.v[j]);
+      } else {
+        for (int i = tid; i < 32 * row8; i += 64 * kLatWaves) k_store(i, k_piece(i, kb));
+        for (int i = tid; i < rank * 4; i += 64 * kLatWaves) v_store(i, v_piece(i, kb));
       }
       __syncthreads();
+      if constexpr (KS > 0) {
+        if (kb + 32 < group_len) st = fetch(kb + 32);         // (the same for all: no barrier inside)
+      }
       if (!mine || kb >= len) continue;
       // ---- scores
       floatx4 s[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
@@ -582,6 +619,7 @@ static void launch_latent_mfma(const void* q, void* out, const void* cache, cons
                                const int* block_table, int max_pages, int page_size, int n, int H, int row, int rank,
                                float scale, float* part, int nslices, hipStream_t stream) {
   const size_t lds = (size_t)(kLatWaves - 1) * (NR * 4 + 2) * kWave * sizeof(float);
+  const unsigned page_magic = (unsigned)(((1ull << 35) + page_size - 1) / page_size);
   static int raised = 0;
   if (lds > 64 * 1024 && !raised) {
     (void)hipFuncSetAttribute((const void*)attn_latent_mfma_kernel<NR, KS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -596,12 +634,12 @@ static void launch_latent_mfma(const void* q, void* out, const void* cache, cons
     }
     hipLaunchKernelGGL((attn_latent_block_kernel<NR, KS>), dim3((n + kLatWaves - 1) / kLatWaves, (H + 15) / 16), dim3(64 * kLatWaves),
                        tiles, stream, (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, positions, span_of_token,
-                       block_table, max_pages, page_size, n, H, row, rank, scale);
+                       block_table, max_pages, page_size, page_magic, n, H, row, rank, scale);
     return;
   }
   hipLaunchKernelGGL((attn_latent_mfma_kernel<NR, KS>), dim3(n, (H + 15) / 16, nslices), dim3(64 * kLatWaves), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, positions, span_of_token, block_table, max_pages,
-                     page_size, H, row, rank, scale, part);
+                     page_size, page_magic, H, row, rank, scale, part);
   if (nslices > 1)
     hipLaunchKernelGGL(attn_latent_merge_kernel, dim3(n * H), dim3(kLatThreads), 0, stream, part, (bf16_t*)out, rank, nslices);
 }
@@ -801,6 +839,7 @@ extern "C" int kllm_attn_latent(const void* q, void* out, const void* cache, con
   KLLM_REQUIRE(max_pages > 0 && page_size > 0, "attn_latent: bad cache sizes");
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "attn_latent: unknown dtype %d", dtype);
   if (dtype == DT_BF16 && mode != 1 && rank % 16 == 0 && row % 8 == 0 && rank <= 512 && page_size % 16 == 0 &&
+      page_size <= 2048 && (long)max_pages * page_size <= (1L << 24) &&
       ((uintptr_t)q & 15) == 0 && ((uintptr_t)cache & 15) == 0 && ((uintptr_t)out & 7) == 0) {
     KLLM_REQUIRE(nslices >= 0 && nslices <= 64 && (nslices <= 1 || (part && part_floats >= (long)n * H * nslices * (rank + 2))),
                  "attn_latent: %d slices need room for %d tokens x %d heads x %d slices x (%d + 2) floats", nslices, n, H,
