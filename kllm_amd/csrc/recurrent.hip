@@ -218,11 +218,12 @@ __global__ __launch_bounds__(kRecThreads) void gated_delta_scan_kernel(
 // ---------------------------------------------------------------------------- gated linear recurrence
 
 constexpr int kGateTokens = 8;       // tokens of a tile of the gates' products
+constexpr int kGateOuts = kRecThreads / 4;   // output channels of a workgroup
 
-// proj: [nsplit][n][2 W], columns y | x.  Workgroup (tile of tokens, block b of the gates): the
-// convolved inputs of the block's channels for the tile's tokens go into LDS [TT][bs]; a thread
-// takes output channel o of the block for all the tile's tokens, the gates' matrices are read
-// [block][in][out] so that neighbouring threads read neighbouring weights.
+// proj: [nsplit][n][2 W], columns y | x.  Workgroup (tile of tokens, block b of the gates, 64 of
+// its output channels): the convolved inputs of the block's channels for the tile's tokens go
+// into LDS [TT][bs]; the gates' matrices are read [block][in][out] so that neighbouring threads
+// read neighbouring weights.
 __global__ __launch_bounds__(kRecThreads) void linear_recurrence_prep_kernel(
     const float* __restrict__ proj, int nsplit, long split_stride, const float* __restrict__ x_bias,
     const float* __restrict__ conv_w, const float* __restrict__ conv_b, int taps, const float* __restrict__ state,
@@ -248,11 +249,20 @@ __global__ __launch_bounds__(kRecThreads) void linear_recurrence_prep_kernel(
   __syncthreads();
   const float* wr = wr_t + (long)b * bs * bs;
   const float* wi = wi_t + (long)b * bs * bs;
-  for (int o = tid; o < bs; o += kRecThreads) {
-    float ar[kGateTokens], ai[kGateTokens];
+  // A workgroup takes kGateOuts output channels (blockIdx.z); four threads share an output, a
+  // quarter of the inputs each, and meet in LDS: a chain of bs / 4 multiply-adds, and four times
+  // the workgroups, where a decode step has one tile of tokens.
+  __shared__ float red[3][kGateOuts][2 * kGateTokens];
+  const int ol = tid % kGateOuts, part = tid / kGateOuts;
+  const int o = blockIdx.z * kGateOuts + ol;
+  const bool o_ok = o < bs;
+  const int per = (bs + 3) / 4, i0 = part * per, i1 = min(bs, i0 + per);
+  float ar[kGateTokens], ai[kGateTokens];
 #pragma unroll
-    for (int tt = 0; tt < kGateTokens; ++tt) ar[tt] = ai[tt] = 0.f;
-    for (int i = 0; i < bs; ++i) {
+  for (int tt = 0; tt < kGateTokens; ++tt) ar[tt] = ai[tt] = 0.f;
+  if (o_ok) {
+#pragma unroll 4
+    for (int i = i0; i < i1; ++i) {
       const float r = wr[(long)i * bs + o], g = wi[(long)i * bs + o];
 #pragma unroll
       for (int tt = 0; tt < kGateTokens; ++tt) {
@@ -261,18 +271,34 @@ __global__ __launch_bounds__(kRecThreads) void linear_recurrence_prep_kernel(
         ai[tt] = fmaf(g, u, ai[tt]);
       }
     }
-    const int c = b * bs + o;
-    const float rb = br[c], ib = bi[c], rt = rate[c];
+  }
+  if (part > 0) {
 #pragma unroll
     for (int tt = 0; tt < kGateTokens; ++tt) {
-      if (tt >= nt) break;
-      const float r = sigmoid_f32(ar[tt] + rb), ig = sigmoid_f32(ai[tt] + ib);
-      const float log_a = -rt * r;
-      const float a = expf(log_a);
-      const float mult = sqrtf(fmaxf(-expm1f(2.f * log_a), 0.f));      // sqrt(1 - a^2)
-      a_out[(tfirst + tt) * W + c] = a;
-      b_out[(tfirst + tt) * W + c] = mult * ig * us[tt * bs + o];
+      red[part - 1][ol][2 * tt] = ar[tt];
+      red[part - 1][ol][2 * tt + 1] = ai[tt];
     }
+  }
+  __syncthreads();
+  if (part > 0 || !o_ok) return;
+#pragma unroll
+  for (int q = 0; q < 3; ++q)          // in a fixed order
+#pragma unroll
+    for (int tt = 0; tt < kGateTokens; ++tt) {
+      ar[tt] += red[q][ol][2 * tt];
+      ai[tt] += red[q][ol][2 * tt + 1];
+    }
+  const int c = b * bs + o;
+  const float rb = br[c], ib = bi[c], rt = rate[c];
+#pragma unroll
+  for (int tt = 0; tt < kGateTokens; ++tt) {
+    if (tt >= nt) break;
+    const float r = sigmoid_f32(ar[tt] + rb), ig = sigmoid_f32(ai[tt] + ib);
+    const float log_a = -rt * r;
+    const float a = expf(log_a);
+    const float mult = sqrtf(fmaxf(-expm1f(2.f * log_a), 0.f));      // sqrt(1 - a^2)
+    a_out[(tfirst + tt) * W + c] = a;
+    b_out[(tfirst + tt) * W + c] = mult * ig * us[tt * bs + o];
   }
 }
 
@@ -448,8 +474,8 @@ extern "C" int kllm_linear_recurrence_prep(const float* proj, int nsplit, long s
   KLLM_REQUIRE(taps >= 1 && taps <= kMaxTaps, "linear_recurrence_prep: %d taps (1 to %d)", taps, kMaxTaps);
   const int bs = W / blocks;
   const size_t lds = (size_t)kGateTokens * bs * sizeof(float);
-  KLLM_REQUIRE(lds <= 64 * 1024, "linear_recurrence_prep: blocks of %d channels do not fit into LDS", bs);
-  hipLaunchKernelGGL(linear_recurrence_prep_kernel, dim3(ceil_div(n, kGateTokens), blocks), dim3(kRecThreads), lds,
+  KLLM_REQUIRE(lds <= 48 * 1024, "linear_recurrence_prep: blocks of %d channels do not fit into LDS", bs);
+  hipLaunchKernelGGL(linear_recurrence_prep_kernel, dim3(ceil_div(n, kGateTokens), blocks, ceil_div(bs, kGateOuts)), dim3(kRecThreads), lds,
                      stream, proj, nsplit, split_stride, x_bias, conv_w, conv_b, taps, state, slot_stride, wr_t, wi_t,
                      br, bi, rate, span_of_token, slots, span_start, span_pos, a_out, b_out, n, W, bs);
   KLLM_CHECK_LAUNCH("linear_recurrence_prep");
