@@ -16,6 +16,9 @@ N4: nothing a multiple of 4 or 8: width 50, five heads of 20 with values of 12, 
 N5: factors of one everywhere (embedding, left and right), kept positions as many as the
     window, a window of one page, heads of 64 on one KV head.
 D1, P1, L1: one mixer each, alone, without feed-forward.
+N6, N7: sizes nearer to a real model's layers (heads of 64 and 128, latents of 160 and 448, delta
+    heads of 64 x 96 and 128 x 128).
+N8: the same delta layer three times, the first two running with the last one's tensors.
 """
 
 import json
