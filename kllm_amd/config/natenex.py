@@ -14,7 +14,7 @@ optional ``mask`` {``size``, ``keep_first``}), ``right`` (a gated linear recurre
 ``blocks``, ``conv``) and the two factors ``left_scale``, ``right_scale``.
 
 ``latent_attention``: ``heads``, ``dim``, ``rot_dim``, ``vdim``, ``q_rank``, ``kv_rank``,
-``scale`` and ``rot`` {``dims``, ``base``}.
+``scale`` and ``rot`` {``dims``, ``base``, optional ``scaling``}.
 
 ``delta``: ``heads``, ``kv_heads``, ``dim``, ``vdim``, ``conv``.
 """
@@ -197,8 +197,6 @@ def _mixer(kind, raw, at):
         rot = _rotation(m.get("rot"), at + ".rot", rot_dim)
         if rot.dims != rot_dim:
             raise ConfigError(f"{at}: rot.dims {rot.dims} is not rot_dim {rot_dim}")
-        if rot.scaling is not None:
-            raise ConfigError(f"{at}.rot: scaled frequencies are not part of this mixer")
         return LatentMixer(m.positive_int("heads"), m.positive_int("dim"), rot_dim, m.positive_int("vdim"),
                            m.positive_int("q_rank"), m.positive_int("kv_rank"), _number(m, "scale"), rot)
     heads, kv = _heads(m, at)

@@ -53,7 +53,8 @@ __device__ __forceinline__ float group4_sum(float v) {
   return v + __shfl_xor(v, 32, kWave);
 }
 
-template <int HDT, int kDecodeWaves, bool BIASED = false>  // head_dim = 16 * HDT; BIASED: scores lose slope * distance
+// KEPT: kept first positions behind the window (an instance of its own: the others carry none of it)
+template <int HDT, int kDecodeWaves, bool BIASED = false, bool KEPT = false>  // head_dim = 16 * HDT; BIASED: scores lose slope * distance
 __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ final_out, float* __restrict__ part,
     const bf16_t* __restrict__ cache,
@@ -76,8 +77,8 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
   const int first = start / 32 * 32;                       // tiles of 32 keys from here
   // Kept first positions: the keys below kept_end (none of them in the window's tiles) come
   // first, in n_kept tiles of their own from key 0; pages between them and the window may be gone.
-  const int kept_end = min(keep_first, first);
-  const int n_kept = (kept_end + 31) / 32;
+  const int kept_end = KEPT ? min(keep_first, first) : 0;
+  const int n_kept = KEPT ? (kept_end + 31) / 32 : 0;
   const int tiles = (len - first + 31) / 32 + n_kept;
   const int per = (tiles + nslices - 1) / nslices;
   const int tile0 = slice * per, tile1 = min(tile0 + per, tiles);
@@ -116,14 +117,16 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
   // Loads carry no branch: a tile or a page that does not exist reads a valid address
   // (table entry 0, page 0) and is marked dead, so that the compiler can count the loads in
   // flight and a tile's arithmetic waits for its own operands only.
-  auto tile_key = [&](int tile) { return tile < n_kept ? tile * 32 : first + (tile - n_kept) * 32; };
+  auto tile_key = [&](int tile) { return (KEPT && tile < n_kept) ? tile * 32 : first + (tile - n_kept) * 32; };
   // a key of tile `tile` is read: below kept_end in a kept tile; in the window, or kept, in the others
   auto key_read = [&](int tile, int key) {
+    if (!KEPT) return key >= start && key < len;
     return tile < n_kept ? key < kept_end : (key < len && (key >= start || key < keep_first));
   };
   auto page_of = [&](int tile, int u) -> int {
     const int k0 = tile_key(tile) + 16 * u;
-    const bool ok = tile < tile1 && (tile < n_kept ? k0 < kept_end : (k0 < len && (k0 + 16 > start || k0 < keep_first)));
+    const bool ok = tile < tile1 && (!KEPT ? (k0 < len && k0 + 16 > start)
+                                           : (tile < n_kept ? k0 < kept_end : (k0 < len && (k0 + 16 > start || k0 < keep_first))));
     const int page = table[ok ? k0 / page_size : 0];
     return ok ? page : -1;
   };
@@ -166,7 +169,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
   }
   auto compute = [&](const Tile& cur, int tile) {
     const int kb = tile_key(tile);
-    const bool edge = tile < n_kept || kb < start || kb + 32 > len;
+    const bool edge = (KEPT && tile < n_kept) || kb < start || kb + 32 > len;
     floatx4 s[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
@@ -321,6 +324,20 @@ static int launch_decode(dim3 grid, hipStream_t stream, const void* q, void* out
                        block_table, max_pages, page_size, H, KV, window, chunk, sink, keep_first, scale, slopes, head_tiles, token_list);
     return 0;
   }
+  if (keep_first > 0) {
+    static int raised_kept = 0;
+    if (lds > 64 * 1024 && !raised_kept) {
+      hipError_t e = hipFuncSetAttribute((const void*)attn_decode_mfma_kernel<HDT, W, false, true>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         W * 16 * (16 * HDT + 4) * (int)sizeof(float));
+      if (e != hipSuccess) KLLM_FAIL((int)e, "attn_decode: cannot raise the LDS limit: %s", hipGetErrorString(e));
+      raised_kept = 1;
+    }
+    hipLaunchKernelGGL((attn_decode_mfma_kernel<HDT, W, false, true>), grid, dim3(64 * W), lds, stream,
+                       (const bf16_t*)q, (bf16_t*)out, part, (const bf16_t*)cache, positions, span_of_token,
+                       block_table, max_pages, page_size, H, KV, window, chunk, sink, keep_first, scale, slopes, head_tiles, token_list);
+    return 0;
+  }
   hipLaunchKernelGGL((attn_decode_mfma_kernel<HDT, W>), grid, dim3(64 * W), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, part, (const bf16_t*)cache, positions, span_of_token,
                      block_table, max_pages, page_size, H, KV, window, chunk, sink, keep_first, scale, slopes, head_tiles, token_list);
@@ -427,6 +444,7 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
   KLLM_REQUIRE(dtype == DT_BF16 || dtype == DT_F32, "%s: unknown dtype %d", who, dtype);
   KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && H % KV == 0, "%s: bad heads n=%d H=%d KV=%d", who, n, H, KV);
   KLLM_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "%s: kept first positions (%d) go with a window", who, keep_first);
+  KLLM_REQUIRE(keep_first == 0 || !slopes, "%s: kept first positions and a distance bias together are not built", who);
   if (dtype == DT_F32) {
     KLLM_REQUIRE(keep_first == 0, "%s: the 32-bit kernels read one run of keys a query", who);
     KLLM_REQUIRE(max_pages > 0 && window >= 0 && chunk >= 0, "%s: bad table width, window or chunk", who);

@@ -474,7 +474,12 @@ extern "C" int kllm_linear_recurrence_prep(const float* proj, int nsplit, long s
   KLLM_REQUIRE(taps >= 1 && taps <= kMaxTaps, "linear_recurrence_prep: %d taps (1 to %d)", taps, kMaxTaps);
   const int bs = W / blocks;
   const size_t lds = (size_t)kGateTokens * bs * sizeof(float);
-  KLLM_REQUIRE(lds <= 48 * 1024, "linear_recurrence_prep: blocks of %d channels do not fit into LDS", bs);
+  KLLM_REQUIRE(lds <= 128 * 1024, "linear_recurrence_prep: blocks of %d channels do not fit into LDS", bs);
+  static size_t raised_to = 48 * 1024;      // beside the kernel's own 12 KB
+  if (lds > raised_to) {
+    (void)hipFuncSetAttribute((const void*)linear_recurrence_prep_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    raised_to = lds;
+  }
   hipLaunchKernelGGL(linear_recurrence_prep_kernel, dim3(ceil_div(n, kGateTokens), blocks, ceil_div(bs, kGateOuts)), dim3(kRecThreads), lds,
                      stream, proj, nsplit, split_stride, x_bias, conv_w, conv_b, taps, state, slot_stride, wr_t, wi_t,
                      br, bi, rate, span_of_token, slots, span_start, span_pos, a_out, b_out, n, W, bs);

@@ -234,7 +234,7 @@ class CausalSelfAttention(Part):
         # the kernels on the matrix cores take keys and values of one width; the 32-bit ones one run of
         # keys a query (no kept first positions)
         fast = (fast and mode != "generic" and self.value_dim == self.head_dim and not self.FAST_KERNELS_OFF
-                and not (self.keep_first and q.dtype != torch.bfloat16))
+                and not (self.keep_first and (q.dtype != torch.bfloat16 or self.slopes is not None)))
         if not fast:
             K.attn_generic(q, out, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
                            cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,

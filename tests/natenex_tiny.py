@@ -46,10 +46,13 @@ def parallel(left, width, blocks, conv, left_scale=1.2, right_scale=0.8, ff=None
                                "left_scale": left_scale, "right_scale": right_scale}, ff, weights_of)
 
 
-def latent(heads, dim, rot_dim, vdim, q_rank, kv_rank, base=10000.0, scale=None, ff=None, weights_of=None):
+def latent(heads, dim, rot_dim, vdim, q_rank, kv_rank, base=10000.0, scale=None, ff=None, weights_of=None, scaling=None):
+    rot = {"base": base, "dims": rot_dim}
+    if scaling:
+        rot["scaling"] = dict(zip(("factor", "low", "high", "original"), scaling))
     return _layer("latent_attention", {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "q_rank": q_rank,
-                                       "kv_rank": kv_rank, "scale": scale or (dim + rot_dim) ** -0.5,
-                                       "rot": {"base": base, "dims": rot_dim}}, ff, weights_of)
+                                       "kv_rank": kv_rank, "scale": scale or (dim + rot_dim) ** -0.5, "rot": rot},
+                  ff, weights_of)
 
 
 def delta(heads, kv, dim, vdim, conv, ff=None, weights_of=None):
@@ -142,7 +145,7 @@ CONFIGS["N6"] = _cfg(200, 192, 1e-6, 1.5, [
     parallel(attn(6, 2, 64, rot=32, base=20000.0, scaling=(8.0, 1.0, 4.0, 64), window=48, keep=4), 256, 8, 4, ff=160,
              weights_of=1)])
 CONFIGS["N7"] = _cfg(160, 128, 1e-5, 0.5, [
-    latent(3, 128, 64, 128, 72, 448, ff=96),
+    latent(3, 128, 64, 128, 72, 448, ff=96, scaling=(2.0, 1.0, 4.0, 40)),
     delta(2, 1, 128, 128, 4),
     parallel(attn(4, 4, 128, vdim=128, rot=128, window=32, keep=1), 128, 2, 2, left_scale=0.5, right_scale=2.0)])
 # The same layer three times, the first of them running with the last one's tensors.
