@@ -41,7 +41,7 @@ def attn(heads, kv, dim, vdim=None, rot=None, base=10000.0, scaling=None, window
     return a
 
 
-def parallel(left, width, blocks, conv, left_scale=1.2, right_scale=0.8, ff=None, weights_of=None):
+def parallel(left, width, blocks, conv, left_scale=1.25, right_scale=0.8, ff=None, weights_of=None):
     return _layer("parallel", {"left": left, "right": {"width": width, "blocks": blocks, "conv": conv},
                                "left_scale": left_scale, "right_scale": right_scale}, ff, weights_of)
 
@@ -140,9 +140,9 @@ def tokens(cfg, n, seed):
 # cached latent rows of several hundred elements, delta heads of 64 and 128.
 CONFIGS["N6"] = _cfg(200, 192, 1e-6, 1.5, [
     delta(6, 3, 64, 96, 4, ff=128),
-    parallel(attn(6, 2, 64, rot=32, base=20000.0, scaling=(8.0, 1.0, 4.0, 64), window=48, keep=4), 256, 8, 4, ff=160),
+    parallel(attn(6, 2, 64, rot=32, base=30000.0, scaling=(6.0, 1.0, 4.0, 64), window=48, keep=4), 256, 8, 4, ff=160),
     latent(6, 64, 32, 64, 96, 160, base=3000.0, ff=128),
-    parallel(attn(6, 2, 64, rot=32, base=20000.0, scaling=(8.0, 1.0, 4.0, 64), window=48, keep=4), 256, 8, 4, ff=160,
+    parallel(attn(6, 2, 64, rot=32, base=30000.0, scaling=(6.0, 1.0, 4.0, 64), window=48, keep=4), 256, 8, 4, ff=160,
              weights_of=1)])
 CONFIGS["N7"] = _cfg(160, 128, 1e-5, 0.5, [
     latent(3, 128, 64, 128, 72, 448, ff=96, scaling=(2.0, 1.0, 4.0, 40)),
