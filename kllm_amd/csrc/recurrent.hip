@@ -169,20 +169,52 @@ __global__ __launch_bounds__(kRecThreads) void gated_delta_scan_kernel(
     s[i] = (col && r < dk && !fresh) ? S[(long)r * dv + j] : 0.f;
   }
   const int QK = G * dk, HV = H * dv;
-  for (long tb = t0; tb < t1; tb += kDeltaBlock) {
-    const int nt = (int)min((long)kDeltaBlock, t1 - tb);
+  // A thread's pieces of a block of tokens: NR elements of k and of q (element i = tid + 256 j of
+  // [TB][dk]), one of v, one of g and beta.  They are asked for one block ahead and wait in
+  // registers while the block before them is multiplied.
+  int tt_of[NR], e_of[NR];
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    const int idx = tid + kRecThreads * i;
+    tt_of[i] = idx < kDeltaBlock * dk ? idx / dk : kDeltaBlock;      // kDeltaBlock: no such element
+    e_of[i] = idx - tt_of[i] * dk;
+  }
+  const int v_tt = tid / kDeltaCols, v_c = blockIdx.z * kDeltaCols + tid % kDeltaCols;
+  struct Pieces {
+    float k[NR], q[NR], v, g;
+  };
+  auto fetch = [&](long tb, int nt) -> Pieces {
+    Pieces P;
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const bool ok = tt_of[i] < nt;
+      const long at = (tb + (ok ? tt_of[i] : 0)) * QK + (long)g * dk + (ok ? e_of[i] : 0);
+      P.k[i] = ok ? kn[at] : 0.f;
+      P.q[i] = ok ? qn[at] : 0.f;
+    }
+    P.v = (v_tt < nt && v_c < dv) ? vv[(tb + v_tt) * HV + (long)h * dv + v_c] : 0.f;
+    P.g = tid < 2 * nt ? gb[(tb + tid / 2) * 2 * H + (tid % 2) * H + h] : 0.f;
+    return P;
+  };
+  long tb = t0;
+  int nt = (int)min((long)kDeltaBlock, t1 - tb);
+  Pieces pre = fetch(tb, nt);
+  while (tb < t1) {
     __syncthreads();                                 // the block before this one has been read
-    for (int i = tid; i < nt * dk; i += kRecThreads) {
-      const int tt = i / dk, e = i % dk;
-      ks[i] = kn[(tb + tt) * QK + (long)g * dk + e];
-      qs[i] = qn[(tb + tt) * QK + (long)g * dk + e];
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const int idx = tid + kRecThreads * i;
+      if (idx < kDeltaBlock * dk) {
+        ks[idx] = pre.k[i];
+        qs[idx] = pre.q[i];
+      }
     }
-    for (int i = tid; i < nt * kDeltaCols; i += kRecThreads) {
-      const int tt = i / kDeltaCols, c = blockIdx.z * kDeltaCols + i % kDeltaCols;
-      vs[i] = c < dv ? vv[(tb + tt) * HV + (long)h * dv + c] : 0.f;
-    }
-    for (int i = tid; i < nt * 2; i += kRecThreads) gs[i] = gb[(tb + i / 2) * 2 * H + (i % 2) * H + h];
+    vs[tid] = pre.v;                                 // [TB][kDeltaCols]: kRecThreads elements
+    if (tid < 2 * kDeltaBlock) gs[tid] = pre.g;
     __syncthreads();
+    const long tb_next = tb + kDeltaBlock;
+    const int nt_next = (int)max(0L, min((long)kDeltaBlock, t1 - tb_next));
+    if (nt_next > 0) pre = fetch(tb_next, nt_next);
     for (int tt = 0; tt < nt; ++tt) {
       const float decay = gs[2 * tt], beta = gs[2 * tt + 1];
       const float* kt = ks + tt * dk;
@@ -207,6 +239,8 @@ __global__ __launch_bounds__(kRecThreads) void gated_delta_scan_kernel(
       o = parts_sum<kDeltaParts>(o);
       if (col && p == 0) o_out[(tb + tt) * HV + (long)h * dv + j] = o;
     }
+    tb = tb_next;
+    nt = nt_next;
   }
 #pragma unroll
   for (int i = 0; i < NR; ++i) {
