@@ -200,6 +200,9 @@ def test_cache_plan_and_kept_first_pages():
     assert kinds.count("paged") == 2 and kinds.count("state") == 2
     windowed = [gp.need for gp in plan.groups if gp.need.kind == "paged" and gp.need.window][0]
     assert (windowed.window, windowed.keep_first) == (24, 3)
+    # the latents: one "head" whose row is the latent and the rotated part, and the latent once more as its values
+    latent = [gp.need for gp in plan.groups if gp.need.kind == "paged" and not gp.need.window][0]
+    assert (latent.kv_heads, latent.head_dim, latent.value_width) == (1, 40 + 8, 40)
     cm = CacheManager([GroupSpec("w", 4, 64, window=10, keep_first=5), GroupSpec("all", 4, 64)], 2)
     cm.open("a")
     cm.reserve("a", 40)
@@ -213,3 +216,16 @@ def test_cache_plan_and_kept_first_pages():
     cm.commit("a", 1)
     cm.release("a")
     assert all(p.free_pages == p.num_pages for p in cm.pools)
+
+
+def test_a_latent_mixer_may_slow_its_rotation_down_too():
+    from kllm_amd.config import config_from_dict
+    raw = copy.deepcopy(T.CONFIGS["L1"])
+    raw["layers"][0]["mixer"]["rot"]["scaling"] = {"factor": 4.0, "low": 1.0, "high": 2.0, "original": 16}
+    cfg = config_from_dict(raw)
+    assert cfg.layers[0].mixer.rot.scaling.factor == 4.0 and cfg.to_dict()["layers"][0]["mixer"]["rot"]["scaling"]["original"] == 16
+    w = P.random_weights(raw, 1)
+    toks = T.tokens(raw, 30, 1)
+    plain = copy.deepcopy(raw)
+    del plain["layers"][0]["mixer"]["rot"]["scaling"]
+    assert (P.forward(raw, w, toks) - P.forward(plain, w, toks)).abs().max() > 1e-3
