@@ -44,8 +44,9 @@ __device__ __forceinline__ float gate_act(float g, int act) {
 
 // Activations without a gate (kllm_unary_act): the gates' two, and xIELU, whose two constants
 // are learned: for z > 0, a_pos z^2 + z/2; otherwise (1/2 + a_neg) (exp(z) - 1 - z) + z/2.
-// The square of the rectifier: max(z, 0)^2.
-enum : int { ACT_XIELU = 2, ACT_TANH = 3, ACT_RELU_SQ = 4, UNARY_ACT_COUNT = 5 };
+// The square of the rectifier: max(z, 0)^2.  The identity (sums that only change their type) and
+// the logistic function.
+enum : int { ACT_XIELU = 2, ACT_TANH = 3, ACT_RELU_SQ = 4, ACT_IDENTITY = 5, ACT_SIGMOID = 6, UNARY_ACT_COUNT = 7 };
 
 __device__ __forceinline__ float softplus_f32(float v) { return v > 20.f ? v : log1pf(expf(v)); }
 
@@ -53,6 +54,8 @@ __device__ __forceinline__ float unary_act(float z, int act, float a_pos, float 
   if (act == ACT_XIELU)
     return z > 0.f ? fmaf(a_pos * z, z, 0.5f * z) : fmaf(0.5f + a_neg, expm1f(z) - z, 0.5f * z);
   if (act == ACT_TANH) return tanhf(z);
+  if (act == ACT_IDENTITY) return z;
+  if (act == ACT_SIGMOID) return 1.f / (1.f + expf(-z));
   if (act == ACT_RELU_SQ) {
     const float p = fmaxf(z, 0.f);
     return p * p;

@@ -60,6 +60,7 @@ static const Op kOps[] = {
     KLLM_CMD_OP(kllm_attn_latent),
     KLLM_CMD_OP(kllm_latent_out),
     KLLM_CMD_OP(kllm_scaled_sum),
+    KLLM_CMD_OP(kllm_normed_sum),
 };
 constexpr int kNumOps = (int)(sizeof(kOps) / sizeof(kOps[0]));
 

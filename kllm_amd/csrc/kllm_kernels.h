@@ -305,18 +305,22 @@ int kllm_group_norm_add(float* x, const float* d1, int ns1, long st1, const floa
                         const int* rows, int n, int d, int groups, float eps, int write_x,
                         hipStream_t stream);
 
-/* Between the query/key product and attention where the values are the keys.  qk holds the
- * sums [nsplit][n][(H + KV) * hd] (queries first).  Biases are added (null: none); the whole
- * query row and the whole key row are each divided by their root mean square (eps inside the
- * root) and multiplied by q_w, k_w (null: no norm); the query is multiplied by
+/* Between the query/key product and attention where queries and keys are normalised over the
+ * whole projection.  qk holds the sums [nsplit][n][(H + KV) * hd + KV * dv] (queries, keys,
+ * values).  Biases are added (null: none); the whole query row and the whole key row are each
+ * divided by their root mean square (eps inside the root) and multiplied by q_w, k_w (null: no
+ * norm); the first `rot` elements of every query and key head then turn (cos/sin [n][rot/2] or
+ * null; pairs (2j, 2j+1) if `interleaved`, else (j, j + rot/2)); the query is multiplied by
  * 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) (temp_every 0: not); q_out
- * [n][H*hd] is written, and into the pages of `cache` (null: no append) go the normalised key
- * as the key and the key before its norm (bias added) as the value. */
+ * [n][H*hd] is written, and into the pages of `cache` (null: no append; keys [KV][slot][hd], then
+ * values [KV][dv][slot]) go the key and the value; with dv == 0 the values are the keys: the key
+ * before its norm (bias added) is cached as the value. */
 int kllm_qk_norm_append(const float* qk, int nsplit, long split_stride, const float* q_bias,
                         const float* k_bias, const float* q_w, const float* k_w, float eps, float temp_coef,
                         int temp_every, void* q_out, void* cache, const int* positions,
                         const int* span_of_token, const int* block_table, int max_pages, int page_size,
-                        int n, int H, int KV, int hd, int dtype, hipStream_t stream);
+                        int n, int H, int KV, int hd, int dtype, int dv, const float* cos_t, const float* sin_t,
+                        int rot, int interleaved, hipStream_t stream);
 
 /* A recurrent mixer with a matrix state per head, S_t = diag(w) S - (a u)(u^T S) + k v^T,
  * o = S^T r, u = k / sqrt(sum k^2 + key_eps).
@@ -339,9 +343,11 @@ int kllm_delta_out(const float* o, const float* gate, const float* weight, float
                    int hd, int dtype, hipStream_t stream);
 
 /* Layers whose norm stands behind the sub-layer.  x [n, d] float32.  With sums (`delta`, float32
- * [nsplit][n][d], plus `bias` [d] or null): x += weight * N(delta + bias); without: x = weight *
- * N(x); N(v) = v / sqrt(mean(v^2) + eps).  `out` (or null) receives the new rows of x in
- * `out_dtype`, for the next product.
+ * [nsplit][n][d], plus `bias` [d] or null): x += mult * weight * N(delta + bias); without: x =
+ * weight * N(x); N(v) = v / sqrt(mean(v^2) + eps).  `out` (or null) receives the new rows of x in
+ * `out_dtype`, for the next product; with `next_weight` [d] it receives next_weight * N(x) of the
+ * new rows instead: the norm in front of the next sub-layer.  `delta_scale` [n] (or null) is a
+ * factor per row on delta's slices.
  * The sums may also be those of a routed feed-forward's chosen experts, not yet added up
  * (`chosen_y` [n * top][d], null: none): then the row is the sum over the token's choices of
  * chosen_wgt * (chosen_idx < E ? chosen_y : chosen_x, the feed-forward's input [n][d]) + delta's
@@ -349,7 +355,8 @@ int kllm_delta_out(const float* o, const float* gate, const float* weight, float
 int kllm_norm_residual(float* x, const float* delta, int nsplit, long split_stride, const float* bias,
                        const float* weight, void* out, int out_dtype, int n, int d, float eps,
                        const float* chosen_y, const void* chosen_x, int chosen_x_dtype, const int* chosen_idx,
-                       const float* chosen_wgt, int top, int E, hipStream_t stream);
+                       const float* chosen_wgt, int top, int E, float mult, const float* next_weight,
+                       const float* delta_scale, hipStream_t stream);
 /* cos/sin [n][half] = factor * cos/sin(positions[t] * freq[i]), the angle in double. */
 int kllm_rope_tables_freq(float* cos_t, float* sin_t, const int* positions, const double* freq, int n,
                           int half, double factor, hipStream_t stream);
@@ -373,19 +380,24 @@ int kllm_qkv_norm_append(const float* qkv, int nsplit, long split_stride, const 
 int kllm_gate_bias(const float* gu, int nsplit, long split_stride, const float* bias, void* out,
                    int out_dtype, int n, int f, int act, float limit, float alpha, hipStream_t stream);
 
-/* A routed feed-forward.  route: z float32 sums [nsplit][n][R] of the router over all R experts;
- * idx/wgt [n][top] receive the `top` experts with the largest softmax(z) + correction (null: none)
- * and their softmax scores divided by their sum.  plan: the entries (token * top + choice) whose
+/* A routed feed-forward.  route: z float32 sums [nsplit][n][cols] of the router, the first R of a
+ * row over all R experts; idx/wgt [n][top] receive the `top` experts with the largest score +
+ * correction (null: none) and their scores divided by their sum (`renorm`), times `scale`; the
+ * score is softmax(z) (`scoring` 0) or the logistic function of z (1).  With `groups` > 1 (up to
+ * 64) the experts form that many equal groups of neighbours, a group's score is the sum of its two
+ * largest, and only experts of the `keep` best groups can be chosen.  With `sgate` [n] the sum
+ * behind the experts' (column R) is a gate's: sgate = its logistic function.  plan: the entries (token * top + choice) whose
  * expert is below E, grouped by expert into `sorted`, and `tiles` [max_tiles][3] = (expert, first
  * place in sorted, entries <= tile_rows); tile_rows is kllm_moe_tile_rows() or twice that (the
  * same in plan and expert); max_tiles >= ceil(entries / tile_rows) + E.
  * expert, mode 0: out [entries][m] (dtype) = gated(gate, up) of x [tokens][k] against w [E][2 m][k];
  * mode 1: out [entries][m] float32 = x [entries][k] against w [E][m][k].  combine: out [n][d] =
  * sum over a token's choices of wgt * (expert < E ? y [entries][d] : xin [n][d]) + the slices of
- * `shared` [ns][n][d] (null: none). */
+ * `shared` [ns][n][d] (null: none), each token's times shared_scale [n] (null: one). */
 int kllm_moe_tile_rows(void);
 int kllm_moe_route(const float* z, int nsplit, long split_stride, const float* correction, int n, int R,
-                   int top, int* idx, float* wgt, hipStream_t stream);
+                   int top, int* idx, float* wgt, int scoring, int groups, int keep, float scale, int renorm,
+                   int cols, float* sgate, hipStream_t stream);
 int kllm_moe_plan(const int* idx, int entries, int E, int max_tiles, int tile_rows, int* sorted, int* tiles,
                   hipStream_t stream);
 int kllm_moe_expert(const void* x, const void* w, void* out, const int* sorted, const int* tiles,
@@ -398,7 +410,7 @@ int kllm_moe_expert_rows(const void* x, const void* w, void* out, const int* idx
                          hipStream_t stream);
 int kllm_moe_combine(const float* y, const void* xin, const int* idx, const float* wgt, const float* shared,
                      int ns, long shared_stride, float* out, int n, int d, int top, int E, int dtype,
-                     hipStream_t stream);
+                     const float* shared_scale, hipStream_t stream);
 
 /* out[r] = sampled index of logits[r][:]; temperature/uniform null: greedy. */
 int kllm_sample(int* out, const float* logits, const float* temperature, const float* uniform,
@@ -426,20 +438,28 @@ int kllm_run_commands(const uint64_t* words, long n_words, int* failed, hipStrea
 int kllm_conv_state_update(const float* proj, int nsplit, long split_stride, int cols, int col0, int C,
                            const float* in_bias, float* state, long slot_stride, int taps, const int* slots,
                            const int* span_start, const int* span_pos, int n_spans, hipStream_t stream);
-/* Gated delta rule, what the recurrence reads.  proj columns: q (G dk) | k (G dk) | v (H dv) | b (H) |
- * a (H) | gate (H dv).  conv_w [2 G dk + H dv][taps]; state: the convolution's field.  Writes qn, kn
- * [n][G dk] (unit vectors per head, qn times dk^-1/2), vv [n][H dv], gb [n][2][H] (decay, beta) and
- * gate [n][H dv] = silu of the gate's sums. */
+/* Gated delta rule, what the recurrence reads.  proj columns (`cols` of them): q (G dk) | k (G dk) |
+ * v (H dv) | b (H) | a (H) | gate (H dv) | anything else.  conv_w [2 G dk + H dv][taps]; state: the
+ * convolution's field.  Writes qn, kn [n][G dk] (unit vectors per head, qn times dk^-1/2), vv [n][H dv],
+ * gb [n][2][H] (decay, beta) and gate [n][H dv] = silu of the gate's sums (`gate_sigmoid`: their
+ * logistic function).  With `a_sums` ([a_ns][n][H dk], a_stride between slices) the decay has one
+ * number per head and key channel, exp(-exp(a_log[h]) softplus(a + dt_bias[h][c])), written to `dec`
+ * [n][H dk]; proj then has no a columns.  With `gate_sums` ([g_ns][n][H dv]) the gate's sums are
+ * these and proj has no gate columns. */
 int kllm_gated_delta_prep(const float* proj, int nsplit, long split_stride, const float* conv_w, int taps,
                           const float* state, long slot_stride, const float* a_log, const float* dt_bias,
                           const int* span_of_token, const int* slots, const int* span_start, const int* span_pos,
                           float* qn, float* kn, float* vv, float* gb, float* gate, int n, int H, int G, int dk,
-                          int dv, float unit_eps, hipStream_t stream);
+                          int dv, float unit_eps, int cols, const float* a_sums, int a_ns, long a_stride,
+                          const float* gate_sums, int g_ns, long g_stride, int gate_sigmoid, float* dec,
+                          hipStream_t stream);
 int kllm_gated_delta_max_dim(void);
-/* The recurrence: state [H][dk][dv] per slot, o_out [n][H dv]. */
+/* The recurrence: state [H][dk][dv] per slot, o_out [n][H dv].  `dec` (or null): decays per head and
+ * key channel [n][H dk], which then take the place of gb's decay. */
 int kllm_gated_delta_scan(const float* qn, const float* kn, const float* vv, const float* gb, float* o_out,
                           float* state, long slot_stride, const int* slots, const int* span_start,
-                          const int* span_pos, int n_spans, int H, int G, int dk, int dv, hipStream_t stream);
+                          const int* span_pos, int n_spans, int H, int G, int dk, int dv, const float* dec,
+                          hipStream_t stream);
 /* Gated linear recurrence.  proj columns: y (W) | x (W).  wr_t, wi_t: the gates' block-diagonal matrices
  * [blocks][in][out]; rate [W] = 8 softplus(lambda).  Writes a and the added term, [n][W] each. */
 int kllm_linear_recurrence_prep(const float* proj, int nsplit, long split_stride, const float* x_bias,
@@ -457,6 +477,10 @@ int kllm_linear_recurrence_scan(const float* a_in, const float* b_in, const floa
 /* out[i] = sa * sum over a's slices + sb * sum over b's slices (float32, `count` elements a slice). */
 int kllm_scaled_sum(float* out, const float* a, int na, long stride_a, float sa, const float* b, int nb,
                     long stride_b, float sb, long count, hipStream_t stream);
+/* out [n][d] = sa * wa * N(a) + sb * wb * N(b), row by row, of the float32 sums a [na][n][d] and b
+ * [nb][n][d]; N(v) = v / sqrt(mean(v^2) + eps); wa, wb [d]. */
+int kllm_normed_sum(float* out, const float* a, int na, long stride_a, float sa, const float* wa, const float* b,
+                    int nb, long stride_b, float sb, const float* wb, int n, int d, float eps, hipStream_t stream);
 
 /* ---- attention through low-rank latents (latent.hip): one cached row of rank + dr per token ---- */
 int kllm_latent_max_row(void);

@@ -1,8 +1,10 @@
 // A routed feed-forward (mixture of experts) whose launches depend on the step's shape only:
 // which token goes to which expert stays on the device.
 //
-//   kllm_moe_route    per token: softmax of the router's sums over all experts, the `top` largest
-//                     of (score + correction), their scores divided by their sum
+//   kllm_moe_route    per token: softmax (or the logistic function) of the router's sums over all
+//                     experts, the `top` largest of (score + correction), optionally only among
+//                     the experts of the best groups of neighbours, their scores divided by their
+//                     sum (or not) and times a constant; a shared expert's gate from one more sum
 //   kllm_moe_plan     the (token, choice) entries grouped by expert, and a list of tiles of up to
 //                     64 entries of one expert (a fixed number of tiles, the unused ones empty)
 //   kllm_moe_expert   one tile's product with its expert's weights on the matrix cores (64 rows by
@@ -29,23 +31,70 @@ constexpr int kMaxRouted = 4096;    // experts a router may choose from at most
 
 // One wave per token; a lane takes the experts lane, lane + 64, ...  The largest of a set is
 // found lane by lane and then across the wave, the lower expert winning a tie.
+// scoring 0: s = softmax(z); 1: s = 1 / (1 + exp(-z)).  groups > 1: the experts form `groups` equal
+// groups of neighbours, a group's score is the sum of its two largest s + correction, and only
+// experts of the `keep` best groups (the lower group winning a tie) can be chosen; lane g works
+// out group g's score.  The weights are the chosen s times `scale`, divided by their sum first
+// if `renorm`.  z's rows are `cols` sums long; with `sgate` the sum behind the experts' is a
+// gate's: sgate[t] = 1 / (1 + exp(-z[t][R])).
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ z, int nsplit, long split_stride,
                                                         const float* __restrict__ correction, int n, int R, int top,
-                                                        int* __restrict__ idx, float* __restrict__ wgt) {
+                                                        int* __restrict__ idx, float* __restrict__ wgt, int scoring,
+                                                        int groups, int keep, float scale, int renorm, int cols,
+                                                        float* __restrict__ sgate) {
   const int t = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
   if (t >= n) return;
   auto z_at = [&](int e) {
     float v = 0.f;
-    for (int s = 0; s < nsplit; ++s) v += z[s * split_stride + (long)t * R + e];
+    for (int s = 0; s < nsplit; ++s) v += z[s * split_stride + (long)t * cols + e];
     return v;
   };
-  float m = -INFINITY;
-  for (int e = lane; e < R; e += kWave) m = fmaxf(m, z_at(e));
-  m = wave_max(m);
-  float den = 0.f;
-  for (int e = lane; e < R; e += kWave) den += expf(z_at(e) - m);
-  den = wave_sum(den);
+  float m = 0.f, den = 1.f;
+  if (scoring == 0) {
+    m = -INFINITY;
+    for (int e = lane; e < R; e += kWave) m = fmaxf(m, z_at(e));
+    m = wave_max(m);
+    den = 0.f;
+    for (int e = lane; e < R; e += kWave) den += expf(z_at(e) - m);
+    den = wave_sum(den);
+  }
+  auto score_at = [&](int e) { return scoring == 0 ? expf(z_at(e) - m) / den : 1.f / (1.f + expf(-z_at(e))); };
+  if (sgate && lane == 0) sgate[t] = 1.f / (1.f + expf(-z_at(R)));
+  unsigned long long open_groups = ~0ull;      // bit g: experts of group g can be chosen
+  const int gsize = R / (groups > 1 ? groups : 1);
+  if (groups > 1) {
+    float gscore = -INFINITY;
+    if (lane < groups) {
+      float a = -INFINITY, b = -INFINITY;      // the two largest of the group
+      for (int e = lane * gsize; e < (lane + 1) * gsize; ++e) {
+        const float c = correction ? score_at(e) + correction[e] : score_at(e);
+        if (c > a) {
+          b = a;
+          a = c;
+        } else if (c > b) {
+          b = c;
+        }
+      }
+      gscore = gsize > 1 ? a + b : a;
+    }
+    open_groups = 0;
+    for (int k = 0; k < keep; ++k) {
+      float best = gscore;
+      int who = lane;
+#pragma unroll
+      for (int off = kWave / 2; off > 0; off >>= 1) {
+        const float ob = __shfl_xor(best, off, kWave);
+        const int ow = __shfl_xor(who, off, kWave);
+        if (ob > best || (ob == best && ow < who)) {
+          best = ob;
+          who = ow;
+        }
+      }
+      open_groups |= 1ull << who;
+      if (lane == who) gscore = -INFINITY;
+    }
+  }
   float picked = 0.f;
   float mine[kMaxTop / kWave] = {};
   unsigned long long taken = 0;      // bit i: this lane's expert lane + 64 i is chosen already
@@ -54,7 +103,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     float best_choice = -INFINITY, best_score = 0.f;
     for (int e = lane; e < R; e += kWave) {
       if ((taken >> (e / kWave)) & 1) continue;
-      const float s = expf(z_at(e) - m) / den;
+      if (groups > 1 && !((open_groups >> (e / gsize)) & 1)) continue;
+      const float s = score_at(e);
       const float c = correction ? s + correction[e] : s;
       if (c > best_choice) {
         best_choice = c;
@@ -77,7 +127,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     if (lane == k % kWave) mine[k / kWave] = best_score;      // lane k keeps the k-th score until the sum is known
     picked += best_score;
   }
-  const float inv = 1.f / (picked + 1e-20f);
+  const float inv = renorm ? scale / (picked + 1e-20f) : scale;
   for (int k = lane; k < top; k += kWave) wgt[(long)t * top + k] = mine[k / kWave] * inv;
 }
 
@@ -352,7 +402,8 @@ __global__ __launch_bounds__(256) void moe_gemv_kernel(const T* __restrict__ X, 
 template <typename T>
 __global__ void moe_combine_kernel(const float* __restrict__ y, const T* __restrict__ xin, const int* __restrict__ idx,
                                    const float* __restrict__ wgt, const float* __restrict__ shared, int ns,
-                                   long shared_stride, float* __restrict__ out, long count, int d, int top, int E) {
+                                   long shared_stride, float* __restrict__ out, long count, int d, int top, int E,
+                                   const float* __restrict__ shared_scale) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= count) return;
   const long t = i / d;
@@ -363,8 +414,9 @@ __global__ void moe_combine_kernel(const float* __restrict__ y, const T* __restr
     const float part = idx[entry] < E ? y[entry * d + c] : to_f32(xin[i]);
     v = fmaf(wgt[entry], part, v);
   }
-  for (int s = 0; s < ns; ++s) v += shared[s * shared_stride + i];
-  out[i] = v;
+  float sh = 0.f;
+  for (int s = 0; s < ns; ++s) sh += shared[s * shared_stride + i];
+  out[i] = shared_scale ? fmaf(shared_scale[t], sh, v) : v + sh;
 }
 
 }  // namespace kllm
@@ -374,12 +426,18 @@ using namespace kllm;
 extern "C" int kllm_moe_tile_rows(void) { return kMoeTileRows; }
 
 extern "C" int kllm_moe_route(const float* z, int nsplit, long split_stride, const float* correction, int n, int R,
-                              int top, int* idx, float* wgt, hipStream_t stream) {
+                              int top, int* idx, float* wgt, int scoring, int groups, int keep, float scale, int renorm,
+                              int cols, float* sgate, hipStream_t stream) {
   KLLM_REQUIRE(z && idx && wgt, "moe_route: null pointer");
+  KLLM_REQUIRE((scoring == 0 || scoring == 1) && cols >= R + (sgate ? 1 : 0),
+               "moe_route: scoring %d, or rows of %d sums for %d experts", scoring, cols, R);
+  KLLM_REQUIRE(groups >= 1 && groups <= kWave && R % groups == 0 && keep >= 1 && keep <= groups &&
+                   top <= R / groups * keep,
+               "moe_route: %d groups (up to %d) of which %d are kept, for %d of %d experts", groups, kWave, keep, top, R);
   KLLM_REQUIRE(n > 0 && R > 0 && R <= kMaxRouted && top > 0 && top <= R && top <= kMaxTop && nsplit >= 1,
                "moe_route: bad sizes n=%d experts=%d (up to %d) top=%d (up to %d)", n, R, kMaxRouted, top, kMaxTop);
   hipLaunchKernelGGL(moe_route_kernel, dim3(ceil_div(n, 4)), dim3(256), 0, stream, z, nsplit, split_stride, correction,
-                     n, R, top, idx, wgt);
+                     n, R, top, idx, wgt, scoring, groups, keep, scale, renorm, cols, sgate);
   KLLM_CHECK_LAUNCH("moe_route");
   return 0;
 }
@@ -451,7 +509,7 @@ extern "C" int kllm_moe_expert_rows(const void* x, const void* w, void* out, con
 
 extern "C" int kllm_moe_combine(const float* y, const void* xin, const int* idx, const float* wgt, const float* shared,
                                 int ns, long shared_stride, float* out, int n, int d, int top, int E, int dtype,
-                                hipStream_t stream) {
+                                const float* shared_scale, hipStream_t stream) {
   KLLM_REQUIRE(y && xin && idx && wgt && out, "moe_combine: null pointer");
   KLLM_REQUIRE(n > 0 && d > 0 && top > 0 && E >= 0 && ns >= 0, "moe_combine: bad sizes n=%d d=%d top=%d", n, d, top);
   KLLM_REQUIRE(shared || ns == 0, "moe_combine: slices of a shared expert without its sums");
@@ -460,10 +518,10 @@ extern "C" int kllm_moe_combine(const float* y, const void* xin, const int* idx,
   const dim3 grid(ceil_div(count, 256));
   if (dtype == DT_F32)
     hipLaunchKernelGGL(moe_combine_kernel<float>, grid, dim3(256), 0, stream, y, (const float*)xin, idx, wgt, shared, ns,
-                       shared_stride, out, count, d, top, E);
+                       shared_stride, out, count, d, top, E, shared_scale);
   else
     hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, grid, dim3(256), 0, stream, y, (const bf16_t*)xin, idx, wgt, shared,
-                       ns, shared_stride, out, count, d, top, E);
+                       ns, shared_stride, out, count, d, top, E, shared_scale);
   KLLM_CHECK_LAUNCH("moe_combine");
   return 0;
 }

@@ -1,10 +1,13 @@
-// What lies between the query/key product and attention for a mixer whose values are its
-// keys: biases, an RMS norm over the whole query projection and one over the whole key
-// projection (all heads at once), a query temperature that grows with the position, and the
-// append to the pages.  The key as projected (bias added, before its norm) is cached as the
-// value, its normalised form as the key.  One workgroup per token, all in 32-bit.
+// What lies between the query/key product and attention for a mixer whose queries and keys
+// are normalised over the whole projection: biases, an RMS norm over the whole query
+// projection and one over the whole key projection (all heads at once), a rotation of the
+// first `rot` elements of every head behind the norm, a query temperature that grows with
+// the position, and the append to the pages.  Without values of its own (dv == 0) the key as
+// projected (bias added, before its norm) is cached as the value, its normalised form as the
+// key; with them (dv > 0) the sums hold KV * dv value columns behind the keys.  One workgroup
+// per token, all in 32-bit.
 //
-// Page layout, per page and KV head: keys [slot][hd], values [hd][slot].
+// Page layout: keys [KV][slot][hd], then values [KV][dv][slot] (dv == 0: values as wide as keys).
 #include <math.h>
 
 #include "common.hpp"
@@ -20,11 +23,11 @@ __global__ __launch_bounds__(kQkThreads) void qk_norm_append_kernel(
     const float* __restrict__ k_bias, const float* __restrict__ q_w, const float* __restrict__ k_w, float eps,
     float temp_coef, int temp_every, T* __restrict__ q_out, T* __restrict__ cache, const int* __restrict__ positions,
     const int* __restrict__ span_of_token, const int* __restrict__ block_table, int max_pages, int page_size, int H,
-    int KV, int hd) {
-  extern __shared__ float row[];            // [H*hd + KV*hd] the sums, then as many norm weights
+    int KV, int hd, int dv, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, int interleaved) {
+  extern __shared__ float row[];            // [H*hd + KV*hd + KV*dv] the sums, then as many norm weights
   __shared__ float red[16];
   const int t = blockIdx.x, tid = threadIdx.x;
-  const int qd = H * hd, kd = KV * hd, cols = qd + kd;
+  const int qd = H * hd, kd = KV * hd, cols = qd + kd + KV * dv;
   const float* in = qk + (long)t * cols;
   float* wrow = row + cols;
   float ssq = 0.f, ssk = 0.f;
@@ -39,12 +42,12 @@ __global__ __launch_bounds__(kQkThreads) void qk_norm_append_kernel(
       if (i < cols) {
         if (i < qd) {
           if (q_w) wv[u] = q_w[i];
-        } else if (k_w) {
+        } else if (k_w && i < qd + kd) {
           wv[u] = k_w[i - qd];
         }
         if (i < qd) {
           if (q_bias) v[u] = q_bias[i];
-        } else if (k_bias) {
+        } else if (k_bias && i < qd + kd) {
           v[u] = k_bias[i - qd];
         }
       }
@@ -59,7 +62,7 @@ __global__ __launch_bounds__(kQkThreads) void qk_norm_append_kernel(
     for (int u = 0; u < 8; ++u) {
       const int i = i0 + u * kQkThreads;
       if (i >= cols) continue;
-      if (i < qd) ssq = fmaf(v[u], v[u], ssq); else ssk = fmaf(v[u], v[u], ssk);
+      if (i < qd) ssq = fmaf(v[u], v[u], ssq); else if (i < qd + kd) ssk = fmaf(v[u], v[u], ssk);
       row[i] = v[u];
       wrow[i] = wv[u];
     }
@@ -71,24 +74,49 @@ __global__ __launch_bounds__(kQkThreads) void qk_norm_append_kernel(
   if (temp_every > 0) qmul = 1.f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.f);
   const float rq = q_w ? 1.f / sqrtf(ssq / (float)qd + eps) : 1.f;
   const float rk = k_w ? 1.f / sqrtf(ssk / (float)kd + eps) : 1.f;
+  // Element i of the normalised query (base 0) or key (base qd) projection, turned with its
+  // partner where it lies among the first `rot` elements of its head.
+  const int rhalf = rot / 2;
+  auto normed = [&](int base, int i, float rs, bool weighted) {
+    const float v = row[base + i];
+    return weighted ? v * rs * wrow[base + i] : v;
+  };
+  auto turned = [&](int base, int i, float rs, bool weighted) {
+    const float v = normed(base, i, rs, weighted);
+    const int e = i % hd;
+    if (!cos_t || e >= rot) return v;
+    int j, partner;
+    bool first;
+    if (interleaved) {
+      j = e / 2;
+      first = (e & 1) == 0;
+      partner = first ? i + 1 : i - 1;
+    } else {
+      first = e < rhalf;
+      j = first ? e : e - rhalf;
+      partner = first ? i + rhalf : i - rhalf;
+    }
+    const float o = normed(base, partner, rs, weighted);
+    const float c = cos_t[(long)t * rhalf + j], sn = sin_t[(long)t * rhalf + j];
+    return first ? v * c - o * sn : v * c + o * sn;
+  };
 #pragma unroll 4
-  for (int i = tid; i < qd; i += kQkThreads) {
-    float v = row[i];
-    if (q_w) v = v * rq * wrow[i];
-    q_out[(long)t * qd + i] = from_f32<T>(v * qmul);
-  }
+  for (int i = tid; i < qd; i += kQkThreads)
+    q_out[(long)t * qd + i] = from_f32<T>(turned(0, i, rq, q_w != nullptr) * qmul);
   if (!cache) return;
   const int page = block_table[(long)span_of_token[t] * max_pages + pos / page_size];
   const int slot = pos % page_size;
-  const long block = (long)page_size * hd;
+  const int vw = dv > 0 ? dv : hd;           // a value's width
+  const long kblock = (long)page_size * hd, vblock = (long)page_size * vw;
+  T* page_base = cache + (long)page * KV * (kblock + vblock);
   for (int i = tid; i < kd; i += kQkThreads) {
     const int kvh = i / hd, e = i % hd;
-    const float raw = row[qd + i];
-    const float key = k_w ? raw * rk * wrow[qd + i] : raw;
-    T* kpage = cache + (((long)page * 2 + 0) * KV + kvh) * block;
-    T* vpage = cache + (((long)page * 2 + 1) * KV + kvh) * block;
-    kpage[(long)slot * hd + e] = from_f32<T>(key);
-    vpage[(long)e * page_size + slot] = from_f32<T>(raw);
+    page_base[kvh * kblock + (long)slot * hd + e] = from_f32<T>(turned(qd, i, rk, k_w != nullptr));
+    if (dv == 0) page_base[KV * kblock + kvh * vblock + (long)e * page_size + slot] = from_f32<T>(row[qd + i]);
+  }
+  for (int i = tid; i < KV * dv; i += kQkThreads) {
+    const int kvh = i / dv, e = i % dv;
+    page_base[KV * kblock + kvh * vblock + (long)e * page_size + slot] = from_f32<T>(row[qd + kd + i]);
   }
 }
 
@@ -100,14 +128,18 @@ extern "C" int kllm_qk_norm_append(const float* qk, int nsplit, long split_strid
                                    const float* k_bias, const float* q_w, const float* k_w, float eps, float temp_coef,
                                    int temp_every, void* q_out, void* cache, const int* positions,
                                    const int* span_of_token, const int* block_table, int max_pages, int page_size,
-                                   int n, int H, int KV, int hd, int dtype, hipStream_t stream) {
+                                   int n, int H, int KV, int hd, int dtype, int dv, const float* cos_t,
+                                   const float* sin_t, int rot, int interleaved, hipStream_t stream) {
   KLLM_REQUIRE(qk && q_out && positions, "qk_norm_append: null pointer");
   KLLM_REQUIRE(!cache || (span_of_token && block_table && max_pages > 0 && page_size > 0),
                "qk_norm_append: a cache needs its tables");
   KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && hd > 0 && nsplit >= 1, "qk_norm_append: bad sizes n=%d H=%d KV=%d hd=%d", n,
                H, KV, hd);
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "qk_norm_append: unknown dtype %d", dtype);
-  const size_t lds = 2 * (size_t)(H + KV) * hd * sizeof(float);
+  KLLM_REQUIRE(dv >= 0 && (cos_t == nullptr) == (sin_t == nullptr), "qk_norm_append: dv %d, or cos without sin", dv);
+  KLLM_REQUIRE(!cos_t || (rot > 0 && rot % 2 == 0 && rot <= hd && (interleaved == 0 || interleaved == 1)),
+               "qk_norm_append: rotary dimension %d of a head of %d", rot, hd);
+  const size_t lds = 2 * ((size_t)(H + KV) * hd + (size_t)KV * dv) * sizeof(float);
   KLLM_REQUIRE(lds <= 160 * 1024, "qk_norm_append: %d query and key channels do not fit into LDS", (H + KV) * hd);
   if (lds > 64 * 1024) {
     const void* fn = dtype == DT_F32 ? (const void*)qk_norm_append_kernel<float> : (const void*)qk_norm_append_kernel<bf16_t>;
@@ -117,11 +149,11 @@ extern "C" int kllm_qk_norm_append(const float* qk, int nsplit, long split_strid
   if (dtype == DT_F32)
     hipLaunchKernelGGL(qk_norm_append_kernel<float>, dim3(n), dim3(kQkThreads), lds, stream, qk, nsplit, split_stride,
                        q_bias, k_bias, q_w, k_w, eps, temp_coef, temp_every, (float*)q_out, (float*)cache, positions,
-                       span_of_token, block_table, max_pages, page_size, H, KV, hd);
+                       span_of_token, block_table, max_pages, page_size, H, KV, hd, dv, cos_t, sin_t, rot, interleaved);
   else
     hipLaunchKernelGGL(qk_norm_append_kernel<bf16_t>, dim3(n), dim3(kQkThreads), lds, stream, qk, nsplit, split_stride,
                        q_bias, k_bias, q_w, k_w, eps, temp_coef, temp_every, (bf16_t*)q_out, (bf16_t*)cache, positions,
-                       span_of_token, block_table, max_pages, page_size, H, KV, hd);
+                       span_of_token, block_table, max_pages, page_size, H, KV, hd, dv, cos_t, sin_t, rot, interleaved);
   KLLM_CHECK_LAUNCH("qk_norm_append");
   return 0;
 }

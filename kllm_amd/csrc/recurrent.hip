@@ -84,7 +84,10 @@ __global__ __launch_bounds__(kRecThreads) void conv_state_update_kernel(
 
 // ---------------------------------------------------------------------------- gated delta rule
 
-// proj: [nsplit][n][cols], columns q (G*dk) | k (G*dk) | v (H*dv) | b (H) | a (H) | gate (H*dv).
+// proj: [nsplit][n][cols], columns q (G*dk) | k (G*dk) | v (H*dv) | b (H) | a (H) | gate (H*dv) |
+// whatever else the product made.  With `a_sums` ([a_ns][n][H*dk]) the decay has one number per
+// head and key channel, from sums of their own, and proj has no a columns; with `gate_sums`
+// ([g_ns][n][H*dv]) the gate's sums are their own too and proj has no gate columns.
 // One workgroup a token.  Dynamic LDS: the convolved q, k, v of the token, [2*G*dk + H*dv] floats.
 __global__ __launch_bounds__(kRecThreads) void gated_delta_prep_kernel(
     const float* __restrict__ proj, int nsplit, long split_stride, const float* __restrict__ conv_w, int taps,
@@ -92,12 +95,13 @@ __global__ __launch_bounds__(kRecThreads) void gated_delta_prep_kernel(
     const float* __restrict__ dt_bias, const int* __restrict__ span_of_token, const int* __restrict__ slots,
     const int* __restrict__ span_start, const int* __restrict__ span_pos, float* __restrict__ qn,
     float* __restrict__ kn, float* __restrict__ vv, float* __restrict__ gb, float* __restrict__ gate, int H, int G,
-    int dk, int dv, float unit_eps) {
+    int dk, int dv, float unit_eps, long cols, const float* __restrict__ a_sums, int a_ns, long a_stride,
+    const float* __restrict__ gate_sums, int g_ns, long g_stride, int gate_sigmoid, float* __restrict__ dec) {
   extern __shared__ float vals[];
   const long t = blockIdx.x;
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int QK = G * dk, HV = H * dv, C = 2 * QK + HV;
-  const long cols = (long)C + 2 * H + HV;
+  const int gate_col = C + (a_sums ? H : 2 * H);
   const int span = span_of_token[t];
   const long t0 = span_start[span];
   const bool fresh = span_pos[span] == 0;
@@ -122,17 +126,28 @@ __global__ __launch_bounds__(kRecThreads) void gated_delta_prep_kernel(
   for (int c = tid; c < HV; c += kRecThreads) {
     vv[t * HV + c] = vals[2 * QK + c];
     float g = 0.f;
-    for (int s = 0; s < nsplit; ++s) g += proj[s * split_stride + t * cols + C + 2 * H + c];
-    gate[t * HV + c] = g / (1.f + expf(-g));
+    if (gate_sums)
+      for (int s = 0; s < g_ns; ++s) g += gate_sums[s * g_stride + t * HV + c];
+    else
+      for (int s = 0; s < nsplit; ++s) g += proj[s * split_stride + t * cols + gate_col + c];
+    gate[t * HV + c] = gate_sigmoid ? sigmoid_f32(g) : g / (1.f + expf(-g));
   }
   for (int h = tid; h < H; h += kRecThreads) {
     float b = 0.f, a = 0.f;
     for (int s = 0; s < nsplit; ++s) {
       b += proj[s * split_stride + t * cols + C + h];
-      a += proj[s * split_stride + t * cols + C + H + h];
+      if (!a_sums) a += proj[s * split_stride + t * cols + C + H + h];
     }
-    gb[t * 2 * H + h] = expf(-expf(a_log[h]) * softplus_f32(a + dt_bias[h]));
+    gb[t * 2 * H + h] = a_sums ? 1.f : expf(-expf(a_log[h]) * softplus_f32(a + dt_bias[h]));
     gb[t * 2 * H + H + h] = sigmoid_f32(b);
+  }
+  if (a_sums) {       // one decay per head and key channel; dt_bias has as many entries
+    const int HK = H * dk;
+    for (int c = tid; c < HK; c += kRecThreads) {
+      float a = 0.f;
+      for (int s = 0; s < a_ns; ++s) a += a_sums[s * a_stride + t * HK + c];
+      dec[t * HK + c] = expf(-expf(a_log[c / dk]) * softplus_f32(a + dt_bias[c]));
+    }
   }
 }
 
@@ -143,17 +158,20 @@ constexpr int kDeltaBlock = 16;                              // tokens staged at
 // Thread (j, p): column j of the workgroup's block of value channels, rows p, p + 16, ... of it.
 // A block of tokens' vectors goes through LDS: k and q [TB][dk] each, v [TB][16 columns], g and
 // beta [TB]; the sums over a column's rows are lane exchanges within its sixteen lanes.
-template <int NR>
+// VEC: the decay has one number per head and key channel (`dec` [n][H*dk], staged like the keys)
+// instead of one per head.
+template <int NR, bool VEC>
 __global__ __launch_bounds__(kRecThreads) void gated_delta_scan_kernel(
     const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vv,
     const float* __restrict__ gb, float* __restrict__ o_out, float* __restrict__ state, long slot_stride,
     const int* __restrict__ slots, const int* __restrict__ span_start, const int* __restrict__ span_pos, int H, int G,
-    int dk, int dv) {
+    int dk, int dv, const float* __restrict__ dec) {
   extern __shared__ float lds[];
   float* ks = lds;                                   // [TB][dk]
   float* qs = ks + kDeltaBlock * dk;                 // [TB][dk]
   float* vs = qs + kDeltaBlock * dk;                 // [TB][kDeltaCols]
   float* gs = vs + kDeltaBlock * kDeltaCols;         // [TB][2]
+  float* ds = gs + 2 * kDeltaBlock;                  // [TB][dk] (VEC)
   const int span = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int g = h / (H / G);
   const int jl = tid / kDeltaParts, p = tid % kDeltaParts;
@@ -181,7 +199,7 @@ __global__ __launch_bounds__(kRecThreads) void gated_delta_scan_kernel(
   }
   const int v_tt = tid / kDeltaCols, v_c = blockIdx.z * kDeltaCols + tid % kDeltaCols;
   struct Pieces {
-    float k[NR], q[NR], v, g;
+    float k[NR], q[NR], d[VEC ? NR : 1], v, g;
   };
   auto fetch = [&](long tb, int nt) -> Pieces {
     Pieces P;
@@ -191,6 +209,8 @@ __global__ __launch_bounds__(kRecThreads) void gated_delta_scan_kernel(
       const long at = (tb + (ok ? tt_of[i] : 0)) * QK + (long)g * dk + (ok ? e_of[i] : 0);
       P.k[i] = ok ? kn[at] : 0.f;
       P.q[i] = ok ? qn[at] : 0.f;
+      if constexpr (VEC)
+        P.d[i] = ok ? dec[(tb + tt_of[i]) * (long)H * dk + (long)h * dk + e_of[i]] : 0.f;
     }
     P.v = (v_tt < nt && v_c < dv) ? vv[(tb + v_tt) * HV + (long)h * dv + v_c] : 0.f;
     P.g = tid < 2 * nt ? gb[(tb + tid / 2) * 2 * H + (tid % 2) * H + h] : 0.f;
@@ -207,6 +227,7 @@ __global__ __launch_bounds__(kRecThreads) void gated_delta_scan_kernel(
       if (idx < kDeltaBlock * dk) {
         ks[idx] = pre.k[i];
         qs[idx] = pre.q[i];
+        if constexpr (VEC) ds[idx] = pre.d[i];
       }
     }
     vs[tid] = pre.v;                                 // [TB][kDeltaCols]: kRecThreads elements
@@ -224,7 +245,7 @@ __global__ __launch_bounds__(kRecThreads) void gated_delta_scan_kernel(
       for (int i = 0; i < NR; ++i) {
         const int r = p + kDeltaParts * i;
         kr[i] = r < dk ? kt[r] : 0.f;
-        s[i] *= decay;
+        if constexpr (VEC) s[i] *= r < dk ? ds[tt * dk + r] : 0.f; else s[i] *= decay;
         dot = fmaf(s[i], kr[i], dot);
       }
       dot = parts_sum<kDeltaParts>(dot);
@@ -420,9 +441,50 @@ __global__ void scaled_sum_kernel(float* __restrict__ out, const float* __restri
   out[i] = fmaf(sa, va, sb * vb);
 }
 
+// out = sa * wa * N(sum of a's slices) + sb * wb * N(sum of b's slices), row by row; N(v) = v /
+// sqrt(mean(v^2) + eps).  One workgroup a row; both rows wait in LDS between the two passes.
+__global__ __launch_bounds__(kRecThreads) void normed_sum_kernel(
+    float* __restrict__ out, const float* __restrict__ a, int na, long stride_a, float sa, const float* __restrict__ wa,
+    const float* __restrict__ b, int nb, long stride_b, float sb, const float* __restrict__ wb, int d, float eps) {
+  extern __shared__ float rows_lds[];     // [2][d]
+  __shared__ float red[16];
+  const long r = blockIdx.x;
+  float ssa = 0.f, ssb = 0.f;
+  for (int i = threadIdx.x; i < d; i += kRecThreads) {
+    float va = 0.f, vb = 0.f;
+    for (int s = 0; s < na; ++s) va += a[r * d + i + s * stride_a];
+    for (int s = 0; s < nb; ++s) vb += b[r * d + i + s * stride_b];
+    rows_lds[i] = va;
+    rows_lds[d + i] = vb;
+    ssa = fmaf(va, va, ssa);
+    ssb = fmaf(vb, vb, ssb);
+  }
+  const float ra = sa / sqrtf(block_sum(ssa, red) / (float)d + eps);
+  const float rb = sb / sqrtf(block_sum(ssb, red) / (float)d + eps);
+  for (int i = threadIdx.x; i < d; i += kRecThreads)     // a thread reads back what it wrote itself
+    out[r * d + i] = fmaf(rows_lds[i] * ra, wa[i], rows_lds[d + i] * rb * wb[i]);
+}
+
 }  // namespace kllm
 
 using namespace kllm;
+
+extern "C" int kllm_normed_sum(float* out, const float* a, int na, long stride_a, float sa, const float* wa,
+                               const float* b, int nb, long stride_b, float sb, const float* wb, int n, int d,
+                               float eps, hipStream_t stream) {
+  KLLM_REQUIRE(out && a && b && wa && wb && na >= 1 && nb >= 1 && n > 0 && d > 0, "normed_sum: null pointer or bad sizes");
+  const size_t lds = 2 * (size_t)d * sizeof(float);
+  KLLM_REQUIRE(lds <= 128 * 1024, "normed_sum: rows of %d do not fit into LDS", d);
+  static size_t raised_to = 48 * 1024;
+  if (lds > raised_to) {
+    (void)hipFuncSetAttribute((const void*)normed_sum_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    raised_to = lds;
+  }
+  hipLaunchKernelGGL(normed_sum_kernel, dim3(n), dim3(kRecThreads), lds, stream, out, a, na, stride_a, sa, wa, b, nb,
+                     stride_b, sb, wb, d, eps);
+  KLLM_CHECK_LAUNCH("normed_sum");
+  return 0;
+}
 
 extern "C" int kllm_scaled_sum(float* out, const float* a, int na, long stride_a, float sa, const float* b, int nb,
                                long stride_b, float sb, long count, hipStream_t stream) {
@@ -452,9 +514,15 @@ extern "C" int kllm_gated_delta_prep(const float* proj, int nsplit, long split_s
                                      const float* state, long slot_stride, const float* a_log, const float* dt_bias,
                                      const int* span_of_token, const int* slots, const int* span_start,
                                      const int* span_pos, float* qn, float* kn, float* vv, float* gb, float* gate,
-                                     int n, int H, int G, int dk, int dv, float unit_eps, hipStream_t stream) {
+                                     int n, int H, int G, int dk, int dv, float unit_eps, int cols,
+                                     const float* a_sums, int a_ns, long a_stride, const float* gate_sums, int g_ns,
+                                     long g_stride, int gate_sigmoid, float* dec, hipStream_t stream) {
   KLLM_REQUIRE(proj && conv_w && state && a_log && dt_bias && span_of_token && slots && span_start && span_pos && qn &&
                    kn && vv && gb && gate, "gated_delta_prep: null pointer");
+  KLLM_REQUIRE((a_sums == nullptr) == (dec == nullptr) && (!a_sums || a_ns >= 1) && (!gate_sums || g_ns >= 1),
+               "gated_delta_prep: decays per key channel come with their sums and a place for them");
+  KLLM_REQUIRE(cols >= 2 * G * dk + H * dv + (a_sums ? H : 2 * H) + (gate_sums ? 0 : H * dv),
+               "gated_delta_prep: %d columns do not hold the projections", cols);
   KLLM_REQUIRE(n > 0 && H > 0 && G > 0 && H % G == 0 && dk > 0 && dv > 0 && nsplit >= 1,
                "gated_delta_prep: bad sizes n=%d H=%d G=%d dk=%d dv=%d", n, H, G, dk, dv);
   KLLM_REQUIRE(taps >= 1 && taps <= kMaxTaps, "gated_delta_prep: %d taps (1 to %d)", taps, kMaxTaps);
@@ -462,7 +530,8 @@ extern "C" int kllm_gated_delta_prep(const float* proj, int nsplit, long split_s
   KLLM_REQUIRE(lds <= 64 * 1024, "gated_delta_prep: %zu bytes of a token's channels do not fit into LDS", lds);
   hipLaunchKernelGGL(gated_delta_prep_kernel, dim3(n), dim3(kRecThreads), lds, stream, proj, nsplit, split_stride,
                      conv_w, taps, state, slot_stride, a_log, dt_bias, span_of_token, slots, span_start, span_pos, qn,
-                     kn, vv, gb, gate, H, G, dk, dv, unit_eps);
+                     kn, vv, gb, gate, H, G, dk, dv, unit_eps, (long)cols, a_sums, a_ns, a_stride, gate_sums, g_ns,
+                     g_stride, gate_sigmoid, dec);
   KLLM_CHECK_LAUNCH("gated_delta_prep");
   return 0;
 }
@@ -471,7 +540,7 @@ extern "C" int kllm_gated_delta_max_dim(void) { return 16 * kDeltaParts; }
 
 extern "C" int kllm_gated_delta_scan(const float* qn, const float* kn, const float* vv, const float* gb, float* o_out,
                                      float* state, long slot_stride, const int* slots, const int* span_start,
-                                     const int* span_pos, int n_spans, int H, int G, int dk, int dv,
+                                     const int* span_pos, int n_spans, int H, int G, int dk, int dv, const float* dec,
                                      hipStream_t stream) {
   KLLM_REQUIRE(qn && kn && vv && gb && o_out && state && slots && span_start && span_pos,
                "gated_delta_scan: null pointer");
@@ -480,11 +549,17 @@ extern "C" int kllm_gated_delta_scan(const float* qn, const float* kn, const flo
                16 * kDeltaParts);
   const dim3 grid(n_spans, H, ceil_div(dv, kDeltaCols));
   KLLM_REQUIRE(grid.z <= 65535, "gated_delta_scan: values too wide for the grid");
-  const size_t lds = ((size_t)kDeltaBlock * (2 * dk + kDeltaCols + 2)) * sizeof(float);
+  const size_t lds = ((size_t)kDeltaBlock * ((dec ? 3 : 2) * dk + kDeltaCols + 2)) * sizeof(float);
   const int nr = ceil_div(dk, kDeltaParts);
-#define KLLM_GDS(NR)                                                                                              \
-  hipLaunchKernelGGL(gated_delta_scan_kernel<NR>, grid, dim3(kRecThreads), lds, stream, qn, kn, vv, gb, o_out, \
-                     state, slot_stride, slots, span_start, span_pos, H, G, dk, dv)
+#define KLLM_GDS(NR)                                                                                                   \
+  do {                                                                                                                 \
+    if (dec)                                                                                                           \
+      hipLaunchKernelGGL((gated_delta_scan_kernel<NR, true>), grid, dim3(kRecThreads), lds, stream, qn, kn, vv, gb,    \
+                         o_out, state, slot_stride, slots, span_start, span_pos, H, G, dk, dv, dec);                   \
+    else                                                                                                               \
+      hipLaunchKernelGGL((gated_delta_scan_kernel<NR, false>), grid, dim3(kRecThreads), lds, stream, qn, kn, vv, gb,   \
+                         o_out, state, slot_stride, slots, span_start, span_pos, H, G, dk, dv, dec);                   \
+  } while (0)
   if (nr <= 1) KLLM_GDS(1);
   else if (nr <= 2) KLLM_GDS(2);
   else if (nr <= 4) KLLM_GDS(4);

@@ -1,8 +1,9 @@
 // Per-token steps of layers whose norm stands behind the sub-layer instead of in front of it,
 // and of attention whose queries and keys are normalised after their rotation:
 //
-//   kllm_norm_residual     x += w * N(d + b), or x = w * N(x); N(v) = v / sqrt(mean(v^2) + eps);
-//                          optionally x rounded to the compute dtype for the next product
+//   kllm_norm_residual     x += m * w * N(d + b), or x = w * N(x); N(v) = v / sqrt(mean(v^2) + eps);
+//                          optionally x rounded to the compute dtype for the next product, or
+//                          N(x) times the weight of the norm in front of the next sub-layer
 //   kllm_rope_tables_freq  cos/sin tables from a table of angles per position (any schedule of
 //                          frequencies), times a constant factor
 //   kllm_qkv_norm_append   biases, rotation of the leading elements of every head, unit RMS of
@@ -39,10 +40,11 @@ template <typename TOUT, int PER>
 __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
     float* __restrict__ x, const float* __restrict__ delta, int nsplit, long split_stride,
     const float* __restrict__ bias, const float* __restrict__ w, TOUT* __restrict__ out, int d, float eps,
-    const ChosenSums chosen) {
+    const ChosenSums chosen, float mult, const float* __restrict__ next_w, const float* __restrict__ delta_scale) {
   extern __shared__ float row_lds[];      // [d] (PER == 0)
   __shared__ float red[16];
   const long r = blockIdx.x;
+  const float dscale = delta_scale ? delta_scale[r] : 1.f;      // a factor of the row's delta (a gate of a shared expert)
   float* xr = x + r * d;
   const bool sums = delta || chosen.y;    // otherwise the stream itself is normalised
   auto chosen_at = [&](int i) {
@@ -93,11 +95,16 @@ __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
         }
       }
       if (delta) {
+        float dv[PER];
+#pragma unroll
+        for (int j = 0; j < PER; ++j) dv[j] = 0.f;
         for (int s = 0; s < nsplit; ++s) {
           const float* src = delta + s * split_stride + r * d;
 #pragma unroll
-          for (int j = 0; j < PER; ++j) v[j] += src[at[j]];
+          for (int j = 0; j < PER; ++j) dv[j] += src[at[j]];
         }
+#pragma unroll
+        for (int j = 0; j < PER; ++j) v[j] = fmaf(dscale, dv[j], v[j]);
       }
       if (bias) {
 #pragma unroll
@@ -114,14 +121,27 @@ __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
 #pragma unroll
     for (int j = 0; j < PER; ++j) ss = fmaf(v[j], v[j], ss);
     const float rstd = 1.f / sqrtf(block_sum(ss, red) / (float)d + eps);
+    float ss2 = 0.f;
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
       const int i = threadIdx.x + kRowThreads * j;
-      if (i >= d) continue;
       const float y = v[j] * rstd * wv[j];
-      const float nv = sums ? xv[j] + y : y;
-      xr[i] = nv;
-      if (out) out[r * d + i] = from_f32<TOUT>(nv);
+      v[j] = i < d ? (sums ? fmaf(mult, y, xv[j]) : y) : 0.f;
+      if (i < d) xr[i] = v[j];
+      ss2 = fmaf(v[j], v[j], ss2);
+    }
+    if (!out) return;
+    if (next_w) {       // the norm in front of the next sub-layer, of the row that is still in registers
+#pragma unroll
+      for (int j = 0; j < PER; ++j) wv[j] = next_w[at[j]];
+      const float rstd2 = 1.f / sqrtf(block_sum(ss2, red) / (float)d + eps);
+#pragma unroll
+      for (int j = 0; j < PER; ++j) v[j] = v[j] * rstd2 * wv[j];
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int i = threadIdx.x + kRowThreads * j;
+      if (i < d) out[r * d + i] = from_f32<TOUT>(v[j]);
     }
     return;
   }
@@ -130,8 +150,11 @@ __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
     float v;
     if (sums) {
       v = chosen.y ? chosen_at(i) : 0.f;
-      if (delta)
-        for (int s = 0; s < nsplit; ++s) v += delta[s * split_stride + r * d + i];
+      if (delta) {
+        float dsum = 0.f;
+        for (int s = 0; s < nsplit; ++s) dsum += delta[s * split_stride + r * d + i];
+        v = fmaf(dscale, dsum, v);
+      }
       if (bias) v += bias[i];
     } else {
       v = xr[i];
@@ -141,12 +164,18 @@ __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
   }
   const float total = block_sum(ss, red);
   const float rstd = 1.f / sqrtf(total / (float)d + eps);
+  float ss2 = 0.f;
   for (int i = threadIdx.x; i < d; i += kRowThreads) {    // a thread reads back what it wrote itself
     const float y = row_lds[i] * rstd * w[i];
-    const float v = sums ? xr[i] + y : y;
+    const float v = sums ? fmaf(mult, y, xr[i]) : y;
     xr[i] = v;
-    if (out) out[r * d + i] = from_f32<TOUT>(v);
+    row_lds[i] = v;
+    ss2 = fmaf(v, v, ss2);
+    if (out && !next_w) out[r * d + i] = from_f32<TOUT>(v);
   }
+  if (!out || !next_w) return;
+  const float rstd2 = 1.f / sqrtf(block_sum(ss2, red) / (float)d + eps);
+  for (int i = threadIdx.x; i < d; i += kRowThreads) out[r * d + i] = from_f32<TOUT>(row_lds[i] * rstd2 * next_w[i]);
 }
 
 __global__ void rope_tables_freq_kernel(float* __restrict__ cos_t, float* __restrict__ sin_t,
@@ -303,8 +332,11 @@ using namespace kllm;
 extern "C" int kllm_norm_residual(float* x, const float* delta, int nsplit, long split_stride, const float* bias,
                                   const float* weight, void* out, int out_dtype, int n, int d, float eps,
                                   const float* chosen_y, const void* chosen_x, int chosen_x_dtype, const int* chosen_idx,
-                                  const float* chosen_wgt, int top, int E, hipStream_t stream) {
+                                  const float* chosen_wgt, int top, int E, float mult, const float* next_weight,
+                                  const float* delta_scale, hipStream_t stream) {
   KLLM_REQUIRE(x && weight, "norm_residual: null pointer");
+  KLLM_REQUIRE(!next_weight || out, "norm_residual: the next norm's rows need a place");
+  KLLM_REQUIRE(!delta_scale || delta, "norm_residual: a factor per row goes with sums");
   KLLM_REQUIRE(!chosen_y || (chosen_x && chosen_idx && chosen_wgt && top > 0 && E >= 0 &&
                              (chosen_x_dtype == DT_F32 || chosen_x_dtype == DT_BF16)),
                "norm_residual: the chosen experts' sums come with their input, choices and weights");
@@ -318,7 +350,7 @@ extern "C" int kllm_norm_residual(float* x, const float* delta, int nsplit, long
 #define KLLM_NR(TOUT, PER)                                                                                    \
   hipLaunchKernelGGL((norm_residual_kernel<TOUT, PER>), dim3(n), dim3(kRowThreads),                           \
                      PER ? 0 : (size_t)d * sizeof(float), stream, x, delta, nsplit, split_stride, bias, weight, \
-                     (TOUT*)out, d, eps, chosen)
+                     (TOUT*)out, d, eps, chosen, mult, next_weight, delta_scale)
   const bool bf = out && out_dtype == DT_BF16;
   if (d <= 4 * kRowThreads) {
     if (bf) KLLM_NR(bf16_t, 4); else KLLM_NR(float, 4);

@@ -21,7 +21,7 @@ import torch
 DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
 GEMV_BEST_ROWS = 0         # rows up to which they beat the MFMA kernels in bfloat16: none (a step at 1.1B sizes, one token: 1.036 against 0.963 ms)
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 
 class KernelError(RuntimeError):
@@ -113,16 +113,16 @@ def _declare(lib):
         "kllm_run_commands": [P, L, P, P],
         "kllm_fused_linear_max_parts": [],
         "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F, P, I, I, P],
-        "kllm_norm_residual": [P, P, I, L, P, P, P, I, I, I, F, P, P, I, P, P, I, I, P],
+        "kllm_norm_residual": [P, P, I, L, P, P, P, I, I, I, F, P, P, I, P, P, I, I, F, P, P, P],
         "kllm_rope_tables_freq": [P, P, P, P, I, I, D, P],
         "kllm_qkv_norm_append": [P, I, L, P, P, P, I, I, I, F, P, P, P, P, P, I, I, I, I, I, I, I, I, P, P, P],
         "kllm_gate_bias": [P, I, L, P, P, I, I, I, I, F, F, P],
         "kllm_moe_tile_rows": [],
-        "kllm_moe_route": [P, I, L, P, I, I, I, P, P, P],
+        "kllm_moe_route": [P, I, L, P, I, I, I, P, P, I, I, I, F, I, I, P, P],
         "kllm_moe_plan": [P, I, I, I, I, P, P, P],
         "kllm_moe_expert": [P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
         "kllm_moe_expert_rows": [P, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
-        "kllm_moe_combine": [P, P, P, P, P, I, L, P, I, I, I, I, I, P],
+        "kllm_moe_combine": [P, P, P, P, P, I, L, P, I, I, I, I, I, P, P],
         "kllm_sample": [P, P, P, P, I, I, P],
         "kllm_attn_decode_slices": [I, I, I, I, I, I],
         "kllm_device_cus": [],
@@ -143,18 +143,20 @@ def _declare(lib):
         "kllm_add_sinusoid": [P, P, I, I, D, P],
         "kllm_unary_act": [P, I, L, I, P, I, I, I, I, P, P],
         "kllm_group_norm_add": [P, P, I, L, P, I, L, P, F, P, P, I, P, I, I, I, F, I, P],
-        "kllm_qk_norm_append": [P, I, L, P, P, P, P, F, F, I, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "kllm_qk_norm_append": [P, I, L, P, P, P, P, F, F, I, P, P, P, P, P, I, I, I, I, I, I, I, I, P, P, I, I, P],
         "kllm_delta_prep": [P, I, L, P, P, P, P, I, L, F, F, P, P, I, I, I, I, I, P],
         "kllm_delta_scan_max_dim": [],
         "kllm_delta_scan": [P, P, P, P, P, P, I, I, I, I, P],
         "kllm_delta_out": [P, P, P, F, P, I, I, I, I, P],
         "kllm_conv_state_update": [P, I, L, I, I, I, P, P, L, I, P, P, P, I, P],
-        "kllm_gated_delta_prep": [P, I, L, P, I, P, L, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, P],
+        "kllm_gated_delta_prep": [P, I, L, P, I, P, L, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, P, I, L, P, I, L,
+                                  I, P, P],
         "kllm_gated_delta_max_dim": [],
-        "kllm_gated_delta_scan": [P, P, P, P, P, P, L, P, P, P, I, I, I, I, I, P],
+        "kllm_gated_delta_scan": [P, P, P, P, P, P, L, P, P, P, I, I, I, I, I, P, P],
         "kllm_linear_recurrence_prep": [P, I, L, P, P, P, I, P, L, P, P, P, P, P, P, P, P, P, P, P, I, I, I, P],
         "kllm_linear_recurrence_scan": [P, P, P, I, L, P, P, L, P, P, P, P, I, I, I, P],
         "kllm_scaled_sum": [P, P, I, L, F, P, I, L, F, L, P],
+        "kllm_normed_sum": [P, P, I, L, F, P, P, I, L, F, P, I, I, F, P],
         "kllm_latent_max_row": [],
         "kllm_latent_kv_append": [P, I, L, P, F, P, P, P, P, P, P, I, I, I, I, I, I, L, P],
         "kllm_latent_norm": [P, I, L, L, P, F, P, I, I, I, P],
@@ -183,7 +185,7 @@ LAUNCHING = ("kllm_embed", "kllm_add_rmsnorm", "kllm_rope_tables", "kllm_rope_ap
              "kllm_moe_plan", "kllm_moe_expert", "kllm_moe_expert_rows", "kllm_moe_combine",
              "kllm_conv_state_update", "kllm_gated_delta_prep", "kllm_gated_delta_scan", "kllm_linear_recurrence_prep",
              "kllm_linear_recurrence_scan", "kllm_latent_kv_append", "kllm_latent_norm", "kllm_latent_query", "kllm_attn_latent",
-             "kllm_latent_out", "kllm_scaled_sum")
+             "kllm_latent_out", "kllm_scaled_sum", "kllm_normed_sum")
 DYNAMIC_ARGS = {"kllm_attn_prefill": (19, 20)}     # arguments that may be a StepValue
 STRUCT_ARGS = {"kllm_gemv_plain": (7,), "kllm_gemv_swiglu": (8,), "kllm_gemv_rope_append": (17,),
                "kllm_fused_linear": (2,)}
@@ -1213,8 +1215,9 @@ def add_sinusoid(x, positions, base=10000.0):
             _ptr(positions, "add_sinusoid positions", torch.int32), n, d, float(base), _stream())
 
 
-ACT_XIELU, ACT_TANH, ACT_RELU_SQ = 2, 3, 4
-UNARY_ACTIVATIONS = dict(ACTIVATIONS, xielu=ACT_XIELU, tanh=ACT_TANH, relu2=ACT_RELU_SQ)
+ACT_XIELU, ACT_TANH, ACT_RELU_SQ, ACT_IDENTITY, ACT_SIGMOID = 2, 3, 4, 5, 6
+UNARY_ACTIVATIONS = dict(ACTIVATIONS, xielu=ACT_XIELU, tanh=ACT_TANH, relu2=ACT_RELU_SQ, identity=ACT_IDENTITY,
+                         sigmoid=ACT_SIGMOID)
 
 
 def _splits(t, n, cols, who):
@@ -1285,14 +1288,19 @@ def group_norm_add(x, deltas=(), bias=None, mult=1.0, weight=None, out=None, row
 
 def qk_norm_append(qk, q_out, cache, positions, span_of_token, block_table, page_size, n_heads, n_kv_heads,
                    head_dim, q_bias=None, k_bias=None, q_weight=None, k_weight=None, eps=0.0, temp_coef=0.0,
-                   temp_every=0):
-    """qk: float32 sums [nsplit, n, (H + KV) * hd] of the query and key products.  Adds the
-    biases, normalises the whole query row and the whole key row (RMS, times their weights),
-    scales the query by 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1), writes q_out and
-    appends to the pages: the normalised key as the key, the key before its norm as the value."""
+                   temp_every=0, value_dim=0, cos=None, sin=None, rotary_dim=0, interleaved=False):
+    """qk: float32 sums [nsplit, n, (H + KV) * hd + KV * value_dim] of the query, key and value
+    products.  Adds the biases, normalises the whole query row and the whole key row (RMS, times
+    their weights), turns the first ``rotary_dim`` elements of every head (cos, sin [n, rotary_dim /
+    2]), scales the query by 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1), writes q_out and
+    appends to the pages.  ``value_dim`` 0: the values are the keys (the normalised key is cached
+    as the key, the key before its norm as the value)."""
     n = q_out.shape[0]
     qd, kd = n_heads * head_dim, n_kv_heads * head_dim
-    nsplit, stride = _splits(qk, n, qd + kd, "qk_norm_append")
+    nsplit, stride = _splits(qk, n, qd + kd + n_kv_heads * value_dim, "qk_norm_append")
+    rot = int(rotary_dim) if cos is not None else 0
+    if cos is not None and (tuple(cos.shape) != (n, rot // 2) or tuple(sin.shape) != tuple(cos.shape)):
+        raise KernelError("qk_norm_append: cos/sin shapes do not fit")
     if q_out.shape[1] != qd:
         raise KernelError("qk_norm_append: q_out does not fit")
     for t, size in ((q_bias, qd), (k_bias, kd), (q_weight, qd), (k_weight, kd)):
@@ -1300,7 +1308,8 @@ def qk_norm_append(qk, q_out, cache, positions, span_of_token, block_table, page
             raise KernelError("qk_norm_append: a bias or norm weight does not fit")
     max_pages = 0
     if cache is not None:
-        if tuple(cache.shape[1:]) != (2, n_kv_heads, page_size * head_dim) or cache.dtype != q_out.dtype:
+        if (not paged_cache_fits(cache, n_kv_heads, page_size, head_dim, value_dim or head_dim)
+                or cache.dtype != q_out.dtype):
             raise KernelError(f"qk_norm_append: cache {tuple(cache.shape)} {cache.dtype} does not fit")
         max_pages = block_table.shape[1]
         if span_of_token.numel() < n:
@@ -1315,7 +1324,9 @@ def qk_norm_append(qk, q_out, cache, positions, span_of_token, block_table, page
             _ptr(cache, "qk_norm_append cache", None, True), _ptr(positions, "qk_norm_append positions", torch.int32),
             _ptr(span_of_token, "qk_norm_append span_of_token", torch.int32, True),
             _ptr(block_table, "qk_norm_append block_table", torch.int32, True), max_pages, page_size, n,
-            n_heads, n_kv_heads, head_dim, dtype_code(q_out.dtype), _stream())
+            n_heads, n_kv_heads, head_dim, dtype_code(q_out.dtype), int(value_dim),
+            _ptr(cos, "qk_norm_append cos", F32, True), _ptr(sin, "qk_norm_append sin", F32, True), rot,
+            1 if interleaved else 0, _stream())
 
 
 DELTA_SCAN_FIELDS = 6      # per token and head the recurrence reads r, k, v, w, u, a*u
@@ -1375,21 +1386,25 @@ def delta_out(o, gate, weight, eps, out, heads, head_dim):
 class ChosenSums:
     """What a routed feed-forward leaves for the norm behind it to add up: per token the weighted
     sum over its choices of ``y`` [n * top, d] (float32), or of ``xin`` [n, d] where the chosen
-    expert is an identity (``idx`` >= ``experts``), plus the slices of ``shared`` (or None)."""
+    expert is an identity (``idx`` >= ``experts``), plus the slices of ``shared`` (or None), each
+    token's times ``shared_scale`` [n] (or None: one)."""
 
-    def __init__(self, y, xin, idx, wgt, experts, shared=None):
+    def __init__(self, y, xin, idx, wgt, experts, shared=None, shared_scale=None):
         self.y, self.xin, self.idx, self.wgt, self.experts, self.shared = y, xin, idx, wgt, int(experts), shared
+        self.shared_scale = shared_scale
 
 
-def norm_residual(x, weight, delta=None, bias=None, out=None, eps=0.0):
+def norm_residual(x, weight, delta=None, bias=None, out=None, eps=0.0, mult=1.0, next_weight=None, delta_scale=None):
     """x [n, d] float32 in place.  With ``delta`` (float32 [n, d] or [nsplit, n, d], or a
-    ``ChosenSums``; ``bias`` [d] is added to it): x += weight * N(delta + bias); without: x =
+    ``ChosenSums``; ``bias`` [d] is added to it): x += mult * weight * N(delta + bias); without: x =
     weight * N(x), where N divides a row by sqrt(mean of its squares + eps).  ``out`` [n, d]
-    receives the new x in its own dtype."""
+    receives the new x in its own dtype, or, with ``next_weight`` [d], next_weight * N(new x): the
+    norm in front of the next sub-layer.  ``delta_scale`` [n]: a factor per row on delta."""
     n, d = x.shape
     chosen = None
     if isinstance(delta, ChosenSums):
         chosen, delta = delta, delta.shared
+        delta_scale = chosen.shared_scale if delta_scale is None else delta_scale
         top = chosen.idx.shape[1]
         if (tuple(chosen.y.shape) != (n * top, d) or tuple(chosen.xin.shape) != (n, d)
                 or tuple(chosen.wgt.shape) != (n, top)):
@@ -1397,6 +1412,9 @@ def norm_residual(x, weight, delta=None, bias=None, out=None, eps=0.0):
     nsplit, stride = (1, 0) if delta is None else _splits(delta, n, d, "norm_residual")
     if weight.numel() != d or (bias is not None and bias.numel() != d) or (out is not None and tuple(out.shape) != (n, d)):
         raise KernelError("norm_residual: weight, bias or output does not fit")
+    if (next_weight is not None and (next_weight.numel() != d or out is None)) or (
+            delta_scale is not None and (delta_scale.numel() != n or delta is None)):
+        raise KernelError("norm_residual: the next norm's weight or the rows' factors do not fit")
     F32 = torch.float32
     _launch("kllm_norm_residual", "norm_residual", _ptr(x, "norm_residual x", F32),
             _ptr(delta, "norm_residual delta", F32, True), nsplit, stride, _ptr(bias, "norm_residual bias", F32, True),
@@ -1406,7 +1424,8 @@ def norm_residual(x, weight, delta=None, bias=None, out=None, eps=0.0):
             dtype_code(chosen.xin.dtype) if chosen else DT_F32,
             _ptr(chosen.idx, "norm_residual idx", torch.int32) if chosen else 0,
             _ptr(chosen.wgt, "norm_residual wgt", F32) if chosen else 0, chosen.idx.shape[1] if chosen else 0,
-            chosen.experts if chosen else 0, _stream())
+            chosen.experts if chosen else 0, float(mult), _ptr(next_weight, "norm_residual next weight", F32, True),
+            _ptr(delta_scale, "norm_residual delta scale", F32, True), _stream())
 
 
 def rope_tables_freq(cos, sin, positions, freq, factor=1.0):
@@ -1486,16 +1505,32 @@ def moe_best_tile_rows(entries, experts) -> int:
     return 2 * small if entries >= 2 * small * experts else small
 
 
-def moe_route(z, correction, idx, wgt):
-    """z: float32 sums [nsplit, n, R] of the router; idx int32, wgt float32 [n, top]."""
+MOE_MAX_GROUPS = 64      # groups of experts a router may choose among
+
+
+def moe_route(z, correction, idx, wgt, experts=None, scoring="softmax", groups=1, keep_groups=1, scale=1.0,
+              renormalize=True, shared_gate=None):
+    """z: float32 sums [nsplit, n, cols] of the router, the first ``experts`` (default: all) of a row
+    the experts'; idx int32, wgt float32 [n, top].  ``scoring``: "softmax" or "sigmoid";
+    ``groups`` > 1: only experts of the ``keep_groups`` best of that many equal groups of
+    neighbours are chosen; the weights are the chosen scores, divided by their sum if
+    ``renormalize``, times ``scale``.  ``shared_gate`` [n] receives the logistic function of the
+    sum behind the experts' (column ``experts``)."""
     n, top = idx.shape
-    R = z.shape[-1]
-    nsplit, stride = _splits(z, n, R, "moe_route")
-    if tuple(wgt.shape) != (n, top) or (correction is not None and correction.numel() != R):
+    cols = z.shape[-1]
+    R = cols if experts is None else int(experts)
+    nsplit, stride = _splits(z, n, cols, "moe_route")
+    if scoring not in ("softmax", "sigmoid"):
+        raise KernelError(f"moe_route: scoring {scoring!r} is not built (softmax, sigmoid)")
+    if (tuple(wgt.shape) != (n, top) or (correction is not None and correction.numel() != R)
+            or cols < R + (1 if shared_gate is not None else 0)
+            or (shared_gate is not None and shared_gate.numel() != n)):
         raise KernelError("moe_route: outputs or correction do not fit")
     _launch("kllm_moe_route", "moe_route", _ptr(z, "moe_route z", torch.float32), nsplit, stride,
             _ptr(correction, "moe_route correction", torch.float32, True), n, R, top,
-            _ptr(idx, "moe_route idx", torch.int32), _ptr(wgt, "moe_route wgt", torch.float32), _stream())
+            _ptr(idx, "moe_route idx", torch.int32), _ptr(wgt, "moe_route wgt", torch.float32),
+            0 if scoring == "softmax" else 1, int(groups), int(keep_groups), float(scale), 1 if renormalize else 0,
+            cols, _ptr(shared_gate, "moe_route shared gate", torch.float32, True), _stream())
 
 
 def moe_plan(idx, experts, sorted_entries, tiles, tile_rows=None):
@@ -1539,9 +1574,9 @@ def moe_expert_rows(x, w, out, idx, experts, mode, act=ACT_SILU, limit=0.0, alph
             m, k, int(mode), int(act), float(limit), float(alpha), dtype_code(x.dtype), _stream())
 
 
-def moe_combine(y, xin, idx, wgt, out, experts, shared=None):
+def moe_combine(y, xin, idx, wgt, out, experts, shared=None, shared_scale=None):
     """out [n, d] float32 = sum over choices of wgt * (idx < experts ? y[token * top + choice] : xin[token])
-    + the slices of ``shared`` (float32 [n, d] or [ns, n, d])."""
+    + the slices of ``shared`` (float32 [n, d] or [ns, n, d]), each token's times ``shared_scale`` [n]."""
     n, d = out.shape
     top = idx.shape[1]
     ns, stride = (0, 0)
@@ -1552,7 +1587,8 @@ def moe_combine(y, xin, idx, wgt, out, experts, shared=None):
     _launch("kllm_moe_combine", "moe_combine", _ptr(y, "moe_combine y", torch.float32), _ptr(xin, "moe_combine x"),
             _ptr(idx, "moe_combine idx", torch.int32), _ptr(wgt, "moe_combine wgt", torch.float32),
             _ptr(shared, "moe_combine shared", torch.float32, True), ns, stride,
-            _ptr(out, "moe_combine out", torch.float32), n, d, top, int(experts), dtype_code(xin.dtype), _stream())
+            _ptr(out, "moe_combine out", torch.float32), n, d, top, int(experts), dtype_code(xin.dtype),
+            _ptr(shared_scale if shared is not None else None, "moe_combine shared scale", torch.float32, True), _stream())
 
 
 # ----------------------------------------------------------------------------- recurrent mixers with a short convolution
@@ -1590,18 +1626,28 @@ def gated_delta_max_dim() -> int:
 
 
 def gated_delta_prep(proj, conv_w, taps, state, conv_offset, a_log, dt_bias, span_of_token, slots, span_start, span_pos,
-                     qn, kn, vv, gb, gate, heads, kv_heads, dim, vdim, unit_eps=1e-6):
-    """proj: float32 sums [nsplit, n, 2 G dk + 2 H dv + 2 H] of q | k | v | b | a | gate.  Convolution
-    (conv_w [2 G dk + H dv, taps], its earlier inputs from the state's field at ``conv_offset``) and
-    SiLU of q, k, v; q and k to unit vectors per head, q times dk^-1/2; gb [n, 2, H] = (exp(-exp(a_log)
-    softplus(a + dt_bias)), sigmoid(b)); gate [n, H dv] = silu of the gate's sums."""
+                     qn, kn, vv, gb, gate, heads, kv_heads, dim, vdim, unit_eps=1e-6, a_sums=None, decays=None,
+                     gate_sums=None, gate_sigmoid=False):
+    """proj: float32 sums [nsplit, n, 2 G dk + 2 H dv + 2 H (or more)] of q | k | v | b | a | gate.
+    Convolution (conv_w [2 G dk + H dv, taps], its earlier inputs from the state's field at
+    ``conv_offset``) and SiLU of q, k, v; q and k to unit vectors per head, q times dk^-1/2; gb [n, 2,
+    H] = (exp(-exp(a_log) softplus(a + dt_bias)), sigmoid(b)); gate [n, H dv] = silu (``gate_sigmoid``:
+    the logistic function) of the gate's sums.  With ``a_sums`` (float32 sums [slices, n, H dk]) the
+    decay has one number per head and key channel (dt_bias [H dk]), written to ``decays`` [n, H dk],
+    and proj has no a columns; with ``gate_sums`` ([slices, n, H dv]) proj has no gate columns."""
     n = qn.shape[0]
     QK, HV = kv_heads * dim, heads * vdim
     C = 2 * QK + HV
-    nsplit, stride = _splits(proj, n, C + 2 * heads + HV, "gated_delta_prep")
+    cols = proj.shape[-1]
+    need = C + (heads if a_sums is not None else 2 * heads) + (0 if gate_sums is not None else HV)
+    nsplit, stride = _splits(proj, n, cols, "gated_delta_prep")
     addr, per_slot = _field(state, conv_offset, "gated_delta_prep")
     F32, I32 = torch.float32, torch.int32
-    if (tuple(conv_w.shape) != (C, taps) or a_log.numel() != heads or dt_bias.numel() != heads
+    a_ns, a_st = _splits(a_sums, n, heads * dim, "gated_delta_prep a") if a_sums is not None else (0, 0)
+    g_ns, g_st = _splits(gate_sums, n, HV, "gated_delta_prep gate") if gate_sums is not None else (0, 0)
+    if (tuple(conv_w.shape) != (C, taps) or a_log.numel() != heads or cols < need
+            or dt_bias.numel() != (heads * dim if a_sums is not None else heads)
+            or (a_sums is None) != (decays is None) or (decays is not None and tuple(decays.shape) != (n, heads * dim))
             or tuple(qn.shape) != (n, QK) or tuple(kn.shape) != (n, QK) or tuple(vv.shape) != (n, HV)
             or tuple(gb.shape) != (n, 2, heads) or tuple(gate.shape) != (n, HV)
             or conv_offset + C * (taps - 1) > per_slot or span_of_token.numel() < n):
@@ -1612,18 +1658,22 @@ def gated_delta_prep(proj, conv_w, taps, state, conv_offset, a_log, dt_bias, spa
             _ptr(slots, "gated_delta slots", I32), _ptr(span_start, "gated_delta span_start", I32),
             _ptr(span_pos, "gated_delta span_pos", I32), _ptr(qn, "gated_delta qn", F32), _ptr(kn, "gated_delta kn", F32),
             _ptr(vv, "gated_delta v", F32), _ptr(gb, "gated_delta gb", F32), _ptr(gate, "gated_delta gate", F32), n,
-            int(heads), int(kv_heads), int(dim), int(vdim), float(unit_eps), _stream())
+            int(heads), int(kv_heads), int(dim), int(vdim), float(unit_eps), int(cols),
+            _ptr(a_sums, "gated_delta a sums", F32, True), a_ns, a_st, _ptr(gate_sums, "gated_delta gate sums", F32, True),
+            g_ns, g_st, 1 if gate_sigmoid else 0, _ptr(decays, "gated_delta decays", F32, True), _stream())
 
 
 def gated_delta_scan(qn, kn, vv, gb, o_out, state, offset, slots, span_start, span_pos, n_spans, heads, kv_heads, dim,
-                     vdim):
+                     vdim, decays=None):
     """S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, each request through its state
-    ([heads, dim, vdim] float32 at ``offset`` floats into its slot; zero where a span's position is 0)."""
+    ([heads, dim, vdim] float32 at ``offset`` floats into its slot; zero where a span's position is 0).
+    ``decays`` [n, heads * dim]: g has one number per head and key channel (a row of S each)."""
     n = qn.shape[0]
     addr, per_slot = _field(state, offset, "gated_delta_scan")
     if (tuple(o_out.shape) != (n, heads * vdim) or tuple(vv.shape) != (n, heads * vdim)
             or tuple(qn.shape) != (n, kv_heads * dim) or tuple(kn.shape) != tuple(qn.shape)
             or tuple(gb.shape) != (n, 2, heads) or offset + heads * dim * vdim > per_slot
+            or (decays is not None and tuple(decays.shape) != (n, heads * dim))
             or slots.numel() < n_spans or span_start.numel() < n_spans + 1 or span_pos.numel() < n_spans):
         raise KernelError("gated_delta_scan: shapes do not fit")
     F32, I32 = torch.float32, torch.int32
@@ -1631,7 +1681,7 @@ def gated_delta_scan(qn, kn, vv, gb, o_out, state, offset, slots, span_start, sp
             _ptr(vv, "gated_delta v", F32), _ptr(gb, "gated_delta gb", F32), _ptr(o_out, "gated_delta o", F32), addr,
             per_slot, _ptr(slots, "gated_delta slots", I32), _ptr(span_start, "gated_delta span_start", I32),
             _ptr(span_pos, "gated_delta span_pos", I32), int(n_spans), int(heads), int(kv_heads), int(dim), int(vdim),
-            _stream())
+            _ptr(decays, "gated_delta decays", F32, True), _stream())
 
 
 def linear_recurrence_prep(proj, x_bias, conv_w, conv_b, taps, state, conv_offset, wr_t, wi_t, br, bi, rate,
@@ -1683,6 +1733,20 @@ def scaled_sum(out, a, scale_a, b, scale_b):
     F32 = torch.float32
     _launch("kllm_scaled_sum", "scaled_sum", _ptr(out, "scaled_sum out", F32), _ptr(a, "scaled_sum a", F32), na, sa,
             float(scale_a), _ptr(b, "scaled_sum b", F32), nb, sb, float(scale_b), n * d, _stream())
+
+
+def normed_sum(out, a, scale_a, weight_a, b, scale_b, weight_b, eps):
+    """out [n, d] float32 = scale_a * weight_a * N(a) + scale_b * weight_b * N(b), row by row; a and b
+    are float32 sums [n, d] or [slices, n, d], N(v) = v / sqrt(mean(v^2) + eps)."""
+    n, d = out.shape
+    na, sa = _splits(a, n, d, "normed_sum")
+    nb, sb = _splits(b, n, d, "normed_sum")
+    if weight_a.numel() != d or weight_b.numel() != d:
+        raise KernelError("normed_sum: the norms' weights do not fit")
+    F32 = torch.float32
+    _launch("kllm_normed_sum", "normed_sum", _ptr(out, "normed_sum out", F32), _ptr(a, "normed_sum a", F32), na, sa,
+            float(scale_a), _ptr(weight_a, "normed_sum weight a", F32), _ptr(b, "normed_sum b", F32), nb, sb,
+            float(scale_b), _ptr(weight_b, "normed_sum weight b", F32), n, d, float(eps), _stream())
 
 
 # ----------------------------------------------------------------------------- attention through low-rank latents

@@ -484,3 +484,67 @@ class NormedQueryKeyAttention(CausalSelfAttention):
         out = ctx.buf("attn.out", (n, self.out_dim), dtype)
         self.attend(ctx, q, out, cache)
         return decode_linear(ctx, out, self.w_o, "attn.proj", self._tiled.get("o"))
+
+
+@register_part("mixer", "attention_whole_norm")
+class WholeNormAttention(CausalSelfAttention):
+    """Attention whose queries and keys pass an RMS norm over the whole projection, all heads at
+    once, with plain weights as long as the projection: q = W_q h, k = W_k h, v = W_v h without
+    biases; the first ``rotary_dim`` elements of every query and key head then turn with the
+    position, if there is a position part (it says how); the query is multiplied by 1 + coef *
+    ln(floor((p + 1) / every) + 1) at position p (``q_temp``); the score is (q . k) * ``scale``;
+    mask (``window``, ``chunk``), ``sink`` and the kernels are the base class's; values may have a
+    width of their own.
+
+    Parameters beyond the base class's: ``eps`` (of the two norms), ``q_temp`` (None or a (coef,
+    every) pair).  Tensors: ``<prefix>.{q,k,v,o}.weight``, ``.{q,k}.norm``."""
+    takes_normed = False
+    fills_sink = False
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        if not self.own_kv:
+            raise ValueError("attention_whole_norm: keeps its own keys and values")
+        self.eps = float(self.param("eps"))
+        temp = self.param("q_temp", None)
+        self.temp_coef, self.temp_every = (float(temp[0]), int(temp[1])) if temp else (0.0, 0)
+        if temp and self.temp_every < 1:
+            raise ValueError(f"attention_whole_norm: q_temp every {self.temp_every} must be positive")
+        self.v_dim = self.kv_heads * self.value_dim
+        self.q_norm = self.k_norm = None
+
+    def weight_specs(self):
+        return [WeightSpec(self.tensor_name("q.weight"), (self.q_dim, self.hidden)),
+                WeightSpec(self.tensor_name("k.weight"), (self.kv_dim, self.hidden)),
+                WeightSpec(self.tensor_name("v.weight"), (self.v_dim, self.hidden)),
+                WeightSpec(self.tensor_name("o.weight"), (self.hidden, self.out_dim)),
+                WeightSpec(self.tensor_name("q.norm"), (self.q_dim,), "vector"),
+                WeightSpec(self.tensor_name("k.norm"), (self.kv_dim,), "vector")]
+
+    def bind(self, weights):
+        self._bind_slopes()
+        self.w_in = torch.cat([weights[self.tensor_name(t + ".weight")] for t in ("q", "k", "v")], dim=0).contiguous()
+        self.w_o = weights[self.tensor_name("o.weight")]
+        self.q_norm = weights[self.tensor_name("q.norm")]
+        self.k_norm = weights[self.tensor_name("k.norm")]
+        # second copies for decode batches, in the order that kernel reads them
+        self._tiled = {"in": tiled_copy(self.runtime, self.w_in, K.LINEAR_PARTS),
+                       "o": tiled_copy(self.runtime, self.w_o, K.LINEAR_PARTS)}
+
+    def forward(self, ctx, xn, cache):
+        n = xn.shape[0]
+        dtype = self.runtime.dtype
+        if not cache.write:
+            raise ValueError("attention_whole_norm: the run writes its own cache")
+        qkv = decode_linear(ctx, xn, self.w_in, "attn.qkv", self._tiled.get("in"))
+        q = ctx.buf("attn.q", (n, self.q_dim), dtype)
+        cos = sin = None
+        if self.position is not None and hasattr(self.position, "tables"):
+            cos, sin = self.position.tables(ctx)
+        K.qk_norm_append(qkv, q, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table, cache.page_size,
+                         self.heads, self.kv_heads, self.head_dim, q_weight=self.q_norm, k_weight=self.k_norm,
+                         eps=self.eps, temp_coef=self.temp_coef, temp_every=self.temp_every, value_dim=self.value_dim,
+                         cos=cos, sin=sin, rotary_dim=self.rotary_dim, interleaved=self.interleaved)
+        out = ctx.buf("attn.out", (n, self.out_dim), dtype)
+        self.attend(ctx, q, out, cache)
+        return decode_linear(ctx, out, self.w_o, "attn.proj", self._tiled.get("o"))

@@ -221,3 +221,97 @@ class SublayerNormBlock(Part):
             K.norm_residual(x, self.norm_ff.weight, delta, bias=getattr(self.feed_forward, "out_bias", None), out=out,
                             eps=self.norm_ff.eps)
         return x, None
+
+
+@register_part("block", "sandwich_norm")
+class SandwichNormBlock(Part):
+    """A norm in front of and behind each sub-layer: a = x + mult * NormB1(Mixer(Norm1(x)));
+    x' = a + mult * NormB2(FeedForward(Norm2(a))).  The layer may have no feed-forward.  All four
+    are RMS norms with ``weight`` and ``eps``.  The norm behind a sub-layer is one launch that adds
+    the sums of the sub-layer's last product (and its bias, ``out_bias`` of a part), normalises,
+    adds to the float32 stream and, behind the mixer, also leaves the rows of the norm in front of
+    the feed-forward (the new row is still in registers).  Nothing stays pending behind the layer.
+
+    Parameters: ``layer`` (its ``norm_mixer`` and ``norm_feed_forward`` stand in front, its
+    ``norm_mixer_out`` and ``norm_feed_forward_out`` behind), ``mult`` (default 1)."""
+    records_launches = True
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        layer = self.param("layer")
+        self.mult = float(self.param("mult", 1.0))
+        if layer.norm_mixer is None or layer.norm_mixer_out is None:
+            raise ValueError("sandwich_norm: the mixer has a norm in front of it and one behind it")
+        self.norm_mixer = make_part("norm", layer.norm_mixer, runtime)
+        self.mixer = make_part("mixer", layer.mixer, runtime)
+        self.norm_mixer_out = make_part("norm", layer.norm_mixer_out, runtime)
+        self.feed_forward = self.norm_ff = self.norm_ff_out = None
+        if layer.feed_forward is not None:
+            if layer.norm_feed_forward is None or layer.norm_feed_forward_out is None:
+                raise ValueError("sandwich_norm: the feed-forward has a norm in front of it and one behind it")
+            self.norm_ff = make_part("norm", layer.norm_feed_forward, runtime)
+            self.feed_forward = make_part("feed_forward", layer.feed_forward, runtime)
+            self.norm_ff_out = make_part("norm", layer.norm_feed_forward_out, runtime)
+        for norm in (self.norm_mixer, self.norm_mixer_out, self.norm_ff, self.norm_ff_out):
+            if norm is not None and not (hasattr(norm, "weight") and hasattr(norm, "eps") and getattr(norm, "groups", 1) == 1):
+                raise ValueError("sandwich_norm: its norms are RMS norms with a weight and eps")
+
+    def parts(self):
+        return [p for p in (self.norm_mixer, self.mixer, self.norm_mixer_out, self.norm_ff, self.feed_forward,
+                            self.norm_ff_out) if p is not None]
+
+    def children(self):
+        return self.parts()
+
+    @property
+    def graph_safe(self):
+        return all(p.graph_safe for p in self.parts())
+
+    def weight_specs(self):
+        return [s for p in self.parts() for s in p.weight_specs()]
+
+    def bind(self, weights):
+        for p in self.parts():
+            p.bind(weights)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def read_bytes(self, tokens):
+        out = {}
+        for p in self.parts():
+            out.update(p.read_bytes(tokens))
+        return out
+
+    def flops(self, tokens, keys_read=0.0):
+        return sum(p.flops(tokens, keys_read) for p in self.parts())
+
+    def first_norm(self):
+        return self.norm_mixer
+
+    def forward(self, ctx, x, pending, cache):
+        if pending is not None:
+            raise ValueError("sandwich_norm: the layer in front of it left sums pending, which it has no norm for")
+        xn = call_part(self.norm_mixer, self.norm_mixer.forward, ctx, x)
+        delta = call_part(self.mixer, self.mixer.forward, ctx, xn, cache)
+        behind = self.norm_mixer_out
+        if self.feed_forward is None:
+            K.norm_residual(x, behind.weight, delta, bias=getattr(self.mixer, "out_bias", None), eps=behind.eps,
+                            mult=self.mult)
+            return x, None
+        if self.norm_ff.eps == behind.eps:
+            # the norm in front of the feed-forward in the same launch
+            xn = ctx.buf("xn", tuple(x.shape), self.runtime.dtype)
+            K.norm_residual(x, behind.weight, delta, bias=getattr(self.mixer, "out_bias", None), eps=behind.eps,
+                            mult=self.mult, out=xn, next_weight=self.norm_ff.weight)
+        else:
+            K.norm_residual(x, behind.weight, delta, bias=getattr(self.mixer, "out_bias", None), eps=behind.eps,
+                            mult=self.mult)
+            xn = call_part(self.norm_ff, self.norm_ff.forward, ctx, x)
+        # a routed feed-forward's weighted sum over the chosen experts is taken in the norm's launch
+        more = {"sums_ok": True} if getattr(self.feed_forward, "leaves_chosen_sums", False) else {}
+        delta = call_part(self.feed_forward, self.feed_forward.forward, ctx, xn, **more)
+        behind = self.norm_ff_out
+        K.norm_residual(x, behind.weight, delta, bias=getattr(self.feed_forward, "out_bias", None), eps=behind.eps,
+                        mult=self.mult)
+        return x, None

@@ -166,7 +166,12 @@ class BiasedGatedFeedForward(Part):
     down(act(gate(x) + b_g) * (up(x) + b_u)) + b_d.  The down projection's bias is left to
     whoever adds the output to the stream (``out_bias``).
 
-    Parameters: ``hidden``, ``intermediate``, ``activation`` (a gate's: "silu", "gelu_tanh").
+    With ``bias`` False there are none, and what is left is a gated feed-forward whose gate the
+    products' own epilogues do not know: "clamped_swish" with g' = min(g, limit), u' = clamp(u,
+    -limit, limit) gives down(g' sigmoid(alpha g') (u' + 1)).
+
+    Parameters: ``hidden``, ``intermediate``, ``activation`` (a gate's: "silu", "gelu_tanh",
+    "clamped_swish" with ``limit`` and ``alpha``), ``bias`` (default True).
     Tensors: ``<prefix>.{gate,up,down}.weight`` and ``.bias``."""
     graph_safe = True
     records_launches = True
@@ -176,29 +181,36 @@ class BiasedGatedFeedForward(Part):
         self.hidden = int(self.param("hidden"))
         self.intermediate = int(self.param("intermediate"))
         act = self.param("activation", "silu")
-        if act not in K.ACTIVATIONS:
-            raise ValueError(f"gated_mlp_bias: activation {act!r} is not built (one of {sorted(K.ACTIVATIONS)})")
-        self.act = K.ACTIVATIONS[act]
+        if act not in K.GATES:
+            raise ValueError(f"gated_mlp_bias: activation {act!r} is not built (one of {sorted(K.GATES)})")
+        self.act = K.GATES[act]
+        self.limit = float(self.param("limit", 0.0))
+        self.alpha = float(self.param("alpha", 1.0))
+        self.has_bias = bool(self.param("bias", True))
         self.w_gu = self.w_down = self.bias_gu = self.out_bias = None
         self._tiled = {}
 
     def weight_specs(self):
         f, d = self.intermediate, self.hidden
-        return [WeightSpec(self.tensor_name("gate.weight"), (f, d)), WeightSpec(self.tensor_name("up.weight"), (f, d)),
-                WeightSpec(self.tensor_name("down.weight"), (d, f)),
-                WeightSpec(self.tensor_name("gate.bias"), (f,), "vector"),
-                WeightSpec(self.tensor_name("up.bias"), (f,), "vector"),
-                WeightSpec(self.tensor_name("down.bias"), (d,), "vector")]
+        specs = [WeightSpec(self.tensor_name("gate.weight"), (f, d)), WeightSpec(self.tensor_name("up.weight"), (f, d)),
+                 WeightSpec(self.tensor_name("down.weight"), (d, f))]
+        if self.has_bias:
+            specs += [WeightSpec(self.tensor_name("gate.bias"), (f,), "vector"),
+                      WeightSpec(self.tensor_name("up.bias"), (f,), "vector"),
+                      WeightSpec(self.tensor_name("down.bias"), (d,), "vector")]
+        return specs
 
     def bind(self, weights):
         w = lambda n: weights[self.tensor_name(n)]
         self.w_gu = torch.cat([w("gate.weight"), w("up.weight")], dim=0).contiguous()
-        self.bias_gu = torch.cat([w("gate.bias"), w("up.bias")]).contiguous()
         self.w_down = w("down.weight")
-        self.out_bias = w("down.bias")
+        if self.has_bias:
+            self.bias_gu = torch.cat([w("gate.bias"), w("up.bias")]).contiguous()
+            self.out_bias = w("down.bias")
         self._tiled = {"gu": tiled_copy(self.runtime, self.w_gu, K.LINEAR_PARTS),
                        "down": tiled_copy(self.runtime, self.w_down, K.LINEAR_PARTS)}
 
     def forward(self, ctx, xn):
-        h = gated_hidden(ctx, xn, self.w_gu, self.intermediate, "ffn", self._tiled.get("gu"), self.bias_gu, self.act)
+        h = gated_hidden(ctx, xn, self.w_gu, self.intermediate, "ffn", self._tiled.get("gu"), self.bias_gu, self.act,
+                         self.limit, self.alpha)
         return decode_linear(ctx, h, self.w_down, "ffn.down", self._tiled.get("down"))

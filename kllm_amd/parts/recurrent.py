@@ -12,6 +12,11 @@ beta = sigmoid(W_b h), g = exp(-exp(A_log) softplus(W_a h + dt_bias)), one of ea
 each head's o is divided by its root mean square (``eps``), multiplied by a weight of
 ``value_dim`` that the heads share and by silu(W_g h), and projected by W_o.
 Tensors: ``<prefix>.{q,k,v,b,a,g,o}.weight``, ``.{q,k,v}.conv``, ``.A_log``, ``.dt_bias``, ``.norm``.
+Variants, each a parameter: ``channel_decay``: g has one number per head and key channel (a row
+of S each), g = exp(-exp(A_log_h) softplus(a + dt_bias)) with a and dt_bias ``heads`` x
+``head_dim`` long; ``low_rank``: the decay's and the output gate's projections are products of
+two matrices, W_a2 (W_a1 h) and W_g2 (W_g1 h) (tensors ``.{a1,a2,g1,g2}.weight``; the inner widths
+are the checkpoint's, or ``a_rank`` and ``gate_rank``); ``gate``: "silu" or "sigmoid".
 
 ``linear_recurrence``: a state per channel.  Two branches of ``width`` channels, y = gelu_tanh(W_y
 h + b_y) and u = conv(W_x h + b_x) + b_c; u is cut into ``blocks`` equal parts, each with two
@@ -25,7 +30,8 @@ convolution's inputs of the last ``taps - 1`` positions; it starts from zero at 
 Everything that enters a recurrence besides the projections' sums is 32-bit.
 
 ``mixer_sum``: two mixers side by side on the same input, ``left_scale * left + right_scale *
-right``; each keeps its own cache or state.
+right``; each keeps its own cache or state.  With ``norm_eps`` each output first passes an RMS norm
+over the model's width with a weight of its own.
 """
 
 from __future__ import annotations
@@ -59,6 +65,16 @@ class GatedDeltaMixer(Part):
             raise ValueError(f"gated_delta: {self.heads} heads are not a multiple of {self.kv_heads} key heads")
         if not 1 <= self.taps <= MAX_TAPS:
             raise ValueError(f"gated_delta: a convolution of {self.taps} taps is not built (1 to {MAX_TAPS})")
+        self.channel_decay = bool(self.param("channel_decay", False))
+        self.low_rank = bool(self.param("low_rank", False))
+        self.a_rank = int(self.param("a_rank", None) or -1)
+        self.gate_rank = int(self.param("gate_rank", None) or -1)
+        gate = self.param("gate", "silu")
+        if gate not in ("silu", "sigmoid"):
+            raise ValueError(f"gated_delta: gate {gate!r} is not built (silu, sigmoid)")
+        self.gate_sigmoid = gate == "sigmoid"
+        self.decays = self.heads * self.head_dim if self.channel_decay else self.heads    # numbers of a token's decay
+        self.w_a2 = self.w_g2 = None
         self.qk = self.kv_heads * self.head_dim
         self.hv = self.heads * self.value_dim
         self.channels = 2 * self.qk + self.hv                 # what passes the convolution
@@ -68,29 +84,52 @@ class GatedDeltaMixer(Part):
 
     def weight_specs(self):
         d = self.hidden
-        return [WeightSpec(self.tensor_name("q.weight"), (self.qk, d)), WeightSpec(self.tensor_name("k.weight"), (self.qk, d)),
-                WeightSpec(self.tensor_name("v.weight"), (self.hv, d)), WeightSpec(self.tensor_name("b.weight"), (self.heads, d)),
-                WeightSpec(self.tensor_name("a.weight"), (self.heads, d)), WeightSpec(self.tensor_name("g.weight"), (self.hv, d)),
-                WeightSpec(self.tensor_name("o.weight"), (d, self.hv)),
-                WeightSpec(self.tensor_name("q.conv"), (self.qk, self.taps), "vector"),
-                WeightSpec(self.tensor_name("k.conv"), (self.qk, self.taps), "vector"),
-                WeightSpec(self.tensor_name("v.conv"), (self.hv, self.taps), "vector"),
-                WeightSpec(self.tensor_name("A_log"), (self.heads,), "vector"),
-                WeightSpec(self.tensor_name("dt_bias"), (self.heads,), "vector"),
-                WeightSpec(self.tensor_name("norm"), (self.value_dim,), "vector")]
+        specs = [WeightSpec(self.tensor_name("q.weight"), (self.qk, d)), WeightSpec(self.tensor_name("k.weight"), (self.qk, d)),
+                 WeightSpec(self.tensor_name("v.weight"), (self.hv, d)), WeightSpec(self.tensor_name("b.weight"), (self.heads, d)),
+                 WeightSpec(self.tensor_name("o.weight"), (d, self.hv)),
+                 WeightSpec(self.tensor_name("q.conv"), (self.qk, self.taps), "vector"),
+                 WeightSpec(self.tensor_name("k.conv"), (self.qk, self.taps), "vector"),
+                 WeightSpec(self.tensor_name("v.conv"), (self.hv, self.taps), "vector"),
+                 WeightSpec(self.tensor_name("A_log"), (self.heads,), "vector"),
+                 WeightSpec(self.tensor_name("dt_bias"), (self.decays,), "vector"),
+                 WeightSpec(self.tensor_name("norm"), (self.value_dim,), "vector")]
+        if self.low_rank:
+            specs += [WeightSpec(self.tensor_name("a1.weight"), (self.a_rank, d)),
+                      WeightSpec(self.tensor_name("a2.weight"), (self.decays, self.a_rank)),
+                      WeightSpec(self.tensor_name("g1.weight"), (self.gate_rank, d)),
+                      WeightSpec(self.tensor_name("g2.weight"), (self.hv, self.gate_rank))]
+        else:
+            specs += [WeightSpec(self.tensor_name("a.weight"), (self.decays, d)),
+                      WeightSpec(self.tensor_name("g.weight"), (self.hv, d))]
+        return specs
 
     def bind(self, weights):
         w = lambda n: weights[self.tensor_name(n)]
-        self.w_in = torch.cat([w(t + ".weight") for t in ("q", "k", "v", "b", "a", "g")], dim=0).contiguous()
+        if self.low_rank:
+            # one product for q, k, v, b and the inner halves of the two low-rank projections
+            self.a_rank, self.gate_rank = w("a1.weight").shape[0], w("g1.weight").shape[0]
+            if w("a2.weight").shape[1] != self.a_rank or w("g2.weight").shape[1] != self.gate_rank:
+                raise ValueError("gated_delta: the two halves of a low-rank projection do not fit each other")
+            self.w_in = torch.cat([w(t + ".weight") for t in ("q", "k", "v", "b", "a1", "g1")], dim=0).contiguous()
+            self.w_a2, self.w_g2 = w("a2.weight"), w("g2.weight")
+        elif self.channel_decay:
+            self.w_in = torch.cat([w(t + ".weight") for t in ("q", "k", "v", "b", "g")], dim=0).contiguous()
+            self.w_a2 = w("a.weight")          # its sums are a product of their own
+        else:
+            self.w_in = torch.cat([w(t + ".weight") for t in ("q", "k", "v", "b", "a", "g")], dim=0).contiguous()
         self.w_o = w("o.weight")
         self.conv = torch.cat([w("q.conv"), w("k.conv"), w("v.conv")], dim=0).contiguous()
         self.a_log, self.dt_bias = w("A_log"), w("dt_bias")
         self.norm_weight = w("norm").repeat(self.heads).contiguous()       # per channel of the concatenated heads
         self._tiled = {"in": tiled_copy(self.runtime, self.w_in, K.LINEAR_PARTS),
                        "o": tiled_copy(self.runtime, self.w_o, K.LINEAR_PARTS)}
+        for key, mat in (("a2", self.w_a2), ("g2", self.w_g2)):
+            if mat is not None:
+                self._tiled[key] = tiled_copy(self.runtime, mat, K.LINEAR_PARTS)
 
     def tensors(self):
-        return [self.w_in, self.w_o, self.conv, self.a_log, self.dt_bias, self.norm_weight]
+        return [t for t in (self.w_in, self.w_o, self.conv, self.a_log, self.dt_bias, self.norm_weight, self.w_a2,
+                            self.w_g2) if t is not None]
 
     def cache_need(self):
         return CacheNeed("state", state_shape=(self.state_floats + self.channels * (self.taps - 1),))
@@ -113,15 +152,32 @@ class GatedDeltaMixer(Part):
         gb = ctx.buf("gdelta.gb", (n, 2, self.heads), f32)
         gate = ctx.buf("gdelta.gate", (n, self.hv), f32)
         conv_at = self.state_floats
+        a_sums = gate_sums = decays = None
+        if self.low_rank:
+            # the inner halves' sums in the compute dtype, then the outer halves' products
+            first = self.channels + self.heads
+            a_in = ctx.buf("gdelta.a1", (n, self.a_rank), self.runtime.dtype)
+            g_in = ctx.buf("gdelta.g1", (n, self.gate_rank), self.runtime.dtype)
+            K.unary_act(proj, a_in, K.ACT_IDENTITY, first_column=first)
+            K.unary_act(proj, g_in, K.ACT_IDENTITY, first_column=first + self.a_rank)
+            a_sums = decode_linear(ctx, a_in, self.w_a2, "gdelta.a", self._tiled.get("a2"))
+            gate_sums = decode_linear(ctx, g_in, self.w_g2, "gdelta.g", self._tiled.get("g2"))
+        elif self.channel_decay:
+            a_sums = decode_linear(ctx, xn, self.w_a2, "gdelta.a", self._tiled.get("a2"))
+        if a_sums is not None and not self.channel_decay:
+            raise ValueError("gated_delta: a low-rank decay is one per head and key channel")
+        if self.channel_decay:
+            decays = ctx.buf("gdelta.decays", (n, self.decays), f32)
         K.gated_delta_prep(proj, self.conv, self.taps, cache.state, conv_at, self.a_log, self.dt_bias, ctx.span_of_token,
                            cache.slots, ctx.span_start, ctx.span_pos, qn, kn, vv, gb, gate, self.heads, self.kv_heads,
-                           self.head_dim, self.value_dim, self.unit_eps)
+                           self.head_dim, self.value_dim, self.unit_eps, a_sums=a_sums, decays=decays,
+                           gate_sums=gate_sums, gate_sigmoid=self.gate_sigmoid)
         # (behind the launch that read the earlier inputs: the span's last ones take their place)
         K.conv_state_update(proj, 0, self.channels, self.taps, cache.state, conv_at, cache.slots, ctx.span_start,
                             ctx.span_pos, ctx.n_spans)
         o = ctx.buf("gdelta.o", (n, self.hv), f32)
         K.gated_delta_scan(qn, kn, vv, gb, o, cache.state, 0, cache.slots, ctx.span_start, ctx.span_pos, ctx.n_spans,
-                           self.heads, self.kv_heads, self.head_dim, self.value_dim)
+                           self.heads, self.kv_heads, self.head_dim, self.value_dim, decays=decays)
         out = ctx.buf("gdelta.out", (n, self.hv), self.runtime.dtype)
         K.delta_out(o, gate, self.norm_weight, self.eps, out, self.heads, self.value_dim)
         return decode_linear(ctx, out, self.w_o, "gdelta.o_proj", self._tiled.get("o"))
@@ -207,7 +263,11 @@ class MixerSum(Part):
     Each keeps what it needs between steps in a cache or state of its own (``cache_need`` is the
     list of both needs; the run is handed one view for each, in that order).
 
-    Parameters: ``left``, ``right`` (PartSpecs of mixers), ``left_scale``, ``right_scale``."""
+    With ``norm_eps`` each output first passes an RMS norm over the model's width with a plain
+    weight of its own (tensors ``<prefix>.left.out``, ``.right.out`` [hidden]).
+
+    Parameters: ``left``, ``right`` (PartSpecs of mixers), ``left_scale``, ``right_scale``,
+    ``norm_eps`` (None: no norms), ``hidden`` (with the norms)."""
     records_launches = True
 
     def __init__(self, spec, runtime):
@@ -216,6 +276,10 @@ class MixerSum(Part):
         self.right = make_part("mixer", self.param("right"), runtime)
         self.left_scale = float(self.param("left_scale", 1.0))
         self.right_scale = float(self.param("right_scale", 1.0))
+        eps = self.param("norm_eps", None)
+        self.norm_eps = float(eps) if eps is not None else None
+        self.hidden = int(self.param("hidden")) if self.norm_eps is not None else 0
+        self.left_norm = self.right_norm = None
         for m in (self.left, self.right):
             if isinstance(m.cache_need(), (list, tuple)):
                 raise ValueError("mixer_sum: its two mixers are plain ones")
@@ -228,14 +292,21 @@ class MixerSum(Part):
         return self.left.graph_safe and self.right.graph_safe
 
     def weight_specs(self):
-        return self.left.weight_specs() + self.right.weight_specs()
+        own = []
+        if self.norm_eps is not None:
+            own = [WeightSpec(self.tensor_name("left.out"), (self.hidden,), "vector"),
+                   WeightSpec(self.tensor_name("right.out"), (self.hidden,), "vector")]
+        return self.left.weight_specs() + self.right.weight_specs() + own
 
     def bind(self, weights):
         self.left.bind(weights)
         self.right.bind(weights)
+        if self.norm_eps is not None:
+            self.left_norm = weights[self.tensor_name("left.out")]
+            self.right_norm = weights[self.tensor_name("right.out")]
 
     def tensors(self):
-        return []
+        return [t for t in (self.left_norm, self.right_norm) if t is not None]
 
     def read_bytes(self, tokens):
         out = dict(self.left.read_bytes(tokens))
@@ -258,5 +329,8 @@ class MixerSum(Part):
         left = call_part(self.left, self.left.forward, ctx, xn, take(self.left))
         right = call_part(self.right, self.right.forward, ctx, xn, take(self.right))
         out = ctx.buf("mixer_sum.out", (xn.shape[0], left.shape[-1]), torch.float32)
-        K.scaled_sum(out, left, self.left_scale, right, self.right_scale)
+        if self.norm_eps is not None:
+            K.normed_sum(out, left, self.left_scale, self.left_norm, right, self.right_scale, self.right_norm, self.norm_eps)
+        else:
+            K.scaled_sum(out, left, self.left_scale, right, self.right_scale)
         return out

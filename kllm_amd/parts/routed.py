@@ -16,11 +16,18 @@ Which token goes where stays on the device: the router's choice is grouped by ex
 of rows (a fixed number of tiles for a step's shape, the unused ones empty), so what is launched
 depends on the shape alone and a step can be recorded.
 
+Other routers, each a parameter: ``scoring`` "sigmoid": s = 1 / (1 + exp(-z)) per expert;
+``groups`` > 1: the experts form that many equal groups of neighbours, a group's score is the sum
+of its two largest (s + correction), and only experts of the ``keep_groups`` best groups can be
+chosen; ``renormalize`` False: a_e = s_e; ``weight_scale``: a_e times a constant; ``shared_gate``:
+the shared expert's output is multiplied, token by token, by 1 / (1 + exp(-w_sg . h)).
+
 Parameters: ``hidden``, ``experts``, ``identity`` (0), ``top``, ``intermediate``, ``limit``,
 ``activation`` ("clamped_swish"), ``alpha`` (1.702), ``correction`` (True: the tensor exists),
-``shared_intermediate`` (None: no shared expert), ``shared_limit``.
+``shared_intermediate`` (None: no shared expert), ``shared_limit``, ``scoring`` ("softmax"),
+``groups`` (1), ``keep_groups``, ``renormalize`` (True), ``weight_scale`` (1), ``shared_gate`` (False).
 Tensors: ``<prefix>.router`` [experts + identity, hidden], ``.correction``,
-``.e<i>.{gate,up,down}``, ``.shared.{gate,up,down}``.
+``.e<i>.{gate,up,down}``, ``.shared.{gate,up,down}``, ``.shared.sg`` [1, hidden].
 """
 
 from __future__ import annotations
@@ -58,6 +65,19 @@ class RoutedExperts(Part):
         self.shared_limit = float(self.param("shared_limit", self.limit))
         if self.experts < 1 or self.identity < 0 or not 1 <= self.top <= self.experts + self.identity:
             raise ValueError(f"routed_experts: top {self.top} of {self.experts} + {self.identity} experts")
+        self.scoring = self.param("scoring", "softmax")
+        if self.scoring not in ("softmax", "sigmoid"):
+            raise ValueError(f"routed_experts: scoring {self.scoring!r} is not built (softmax, sigmoid)")
+        self.groups = int(self.param("groups", 1) or 1)
+        self.keep_groups = int(self.param("keep_groups", self.groups) or self.groups)
+        routed = self.experts + self.identity
+        if (self.groups < 1 or self.groups > K.MOE_MAX_GROUPS or routed % self.groups
+                or not 1 <= self.keep_groups <= self.groups or self.top > routed // self.groups * self.keep_groups):
+            raise ValueError(f"routed_experts: {routed} experts in {self.groups} groups (up to {K.MOE_MAX_GROUPS}) of "
+                             f"which {self.keep_groups} are kept, for {self.top} choices")
+        self.renormalize = bool(self.param("renormalize", True))
+        self.weight_scale = float(self.param("weight_scale", 1.0))
+        self.shared_gate = bool(self.param("shared_gate", False)) and bool(shared)
         self.w_router = self.correction = self.w_gu = self.w_down = self.w_shared_gu = self.w_shared_down = None
         self._tiled = {}
 
@@ -76,10 +96,14 @@ class RoutedExperts(Part):
             sf = self.shared_intermediate
             specs += [WeightSpec(self.tensor_name("shared.gate"), (sf, d)), WeightSpec(self.tensor_name("shared.up"), (sf, d)),
                       WeightSpec(self.tensor_name("shared.down"), (d, sf))]
+        if self.shared_gate:
+            specs.append(WeightSpec(self.tensor_name("shared.sg"), (1, d)))
         return specs
 
     def bind(self, weights):
         self.w_router = weights[self.tensor_name("router")]
+        if self.shared_gate:       # the gate's sum is one more of the router's product
+            self.w_router = torch.cat([self.w_router, weights[self.tensor_name("shared.sg")]], dim=0).contiguous()
         self.correction = weights[self.tensor_name("correction")] if self.has_correction else None
         gu, down = [], []
         for e in range(self.experts):
@@ -106,7 +130,7 @@ class RoutedExperts(Part):
 
     def flops(self, tokens, keys_read=0.0):
         d, f = self.hidden, self.intermediate
-        total = 2.0 * tokens * (self.experts + self.identity) * d + 6.0 * tokens * self.top * d * f
+        total = 2.0 * tokens * self.w_router.shape[0] * d + 6.0 * tokens * self.top * d * f
         if self.shared_intermediate:
             total += 6.0 * tokens * d * self.shared_intermediate
         return total
@@ -121,7 +145,10 @@ class RoutedExperts(Part):
         z = decode_linear(ctx, xn, self.w_router, "moe.z", self._tiled.get("router"))
         idx = ctx.buf("moe.idx", (n, top), torch.int32)
         wgt = ctx.buf("moe.wgt", (n, top), torch.float32)
-        K.moe_route(z, self.correction, idx, wgt)
+        sgate = ctx.buf("moe.sgate", (n,), torch.float32) if self.shared_gate else None
+        K.moe_route(z, self.correction, idx, wgt, experts=self.experts + self.identity, scoring=self.scoring,
+                    groups=self.groups, keep_groups=self.keep_groups, scale=self.weight_scale,
+                    renormalize=self.renormalize, shared_gate=sgate)
         h = ctx.buf("moe.h", (n * top, f), dtype)
         y = ctx.buf("moe.y", (n * top, d), torch.float32)
         if n * top <= K.MOE_ROWS_BEST_ENTRIES and not self.runtime.options.get("moe_tiles_only"):
@@ -141,7 +168,7 @@ class RoutedExperts(Part):
                               self._tiled.get("shared_gu"), None, self.act, self.shared_limit, self.alpha)
             shared = decode_linear(ctx, hs, self.w_shared_down, "moe.shared.down", self._tiled.get("shared_down"))
         if sums_ok:
-            return K.ChosenSums(y, xn, idx, wgt, self.experts, shared)
+            return K.ChosenSums(y, xn, idx, wgt, self.experts, shared, sgate)
         out = ctx.buf("moe.out", (n, d), torch.float32)
-        K.moe_combine(y, xn, idx, wgt, out, self.experts, shared)
+        K.moe_combine(y, xn, idx, wgt, out, self.experts, shared, sgate)
         return out

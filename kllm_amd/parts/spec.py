@@ -82,11 +82,15 @@ class PartSpec:
 class LayerSpec:
     """One layer: an arrangement (block kind) of norms, a mixer and a
     feed-forward.  Each layer chooses its own parts; an arrangement that has no
-    use for one of them (one norm for both sub-layers, no feed-forward) leaves it None."""
+    use for one of them (one norm for both sub-layers, no feed-forward) leaves it None.  An
+    arrangement with a norm on both sides of a sub-layer names the ones behind the sub-layers in
+    ``norm_mixer_out`` and ``norm_feed_forward_out``."""
     mixer: PartSpec
     feed_forward: Optional[PartSpec] = None
     norm_mixer: Optional[PartSpec] = None
     norm_feed_forward: Optional[PartSpec] = None
+    norm_mixer_out: Optional[PartSpec] = None
+    norm_feed_forward_out: Optional[PartSpec] = None
     block: str = "pre_norm"
     block_params: Dict[str, Any] = field(default_factory=dict)
 
