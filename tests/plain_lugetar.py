@@ -192,24 +192,36 @@ def expert(h, w, p):
     return (silu(h @ w[p + ".gate"].T) * (h @ w[p + ".up"].T)) @ w[p + ".down"].T
 
 
-def choose_experts(scores, top, groups, keep):
+def choose_experts(scores, top, groups, keep, margin=None):
     """scores [E] -> the ``top`` experts with the largest scores among the experts of the ``keep``
-    best of ``groups`` equal groups of neighbours; a group's score is the sum of its two largest."""
+    best of ``groups`` equal groups of neighbours; a group's score is the sum of its two largest.
+    ``margin`` (a list) receives by how much the closest call was decided: the least kept group's
+    score over the best dropped one's, the least chosen score over the best that was not."""
     E = scores.numel()
     size = E // groups
     allowed = torch.ones(E, dtype=torch.bool)
+    gaps = []
     if groups > 1:
         by_group = scores.reshape(groups, size)
         group_score = by_group.topk(min(2, size), dim=-1).values.sum(-1)
-        kept = group_score.topk(keep).indices
+        ranked = group_score.sort(descending=True)
+        kept = ranked.indices[:keep]
+        if keep < groups:
+            gaps.append(float(ranked.values[keep - 1] - ranked.values[keep]))
         allowed = torch.zeros(groups, size, dtype=torch.bool)
         allowed[kept] = True
         allowed = allowed.reshape(E)
     masked = scores.masked_fill(~allowed, float("-inf"))
-    return masked.topk(top).indices
+    ranked = masked.sort(descending=True)
+    if top < int(allowed.sum()):
+        gaps.append(float(ranked.values[top - 1] - ranked.values[top]))
+    if margin is not None:
+        margin.append(min(gaps) if gaps else float("inf"))
+    return ranked.indices[:top]
 
 
-def moe_ff(h, w, p, mlp):
+def moe_ff(h, w, p, mlp, margins=None):
+    """``margins`` (a list) receives, token by token, by how much the router's closest call was decided."""
     r = mlp["router"]
     E, top, scale = int(r["experts"]), int(r["top"]), float(r.get("scale", 1.0))
     groups = r.get("groups") or {}
@@ -217,7 +229,7 @@ def moe_ff(h, w, p, mlp):
     s = torch.sigmoid(h @ w[p + ".router"].T)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
-        for e in choose_experts(s[t], top, count, keep).tolist():
+        for e in choose_experts(s[t], top, count, keep, margins).tolist():
             out[t] = out[t] + scale * s[t, e] * expert(h[t:t + 1], w, f"{p}.e{e}")[0]
     if mlp.get("shared"):
         out = out + torch.sigmoid(h @ w[p + ".shared.sg"].T) * expert(h, w, p + ".shared")
@@ -226,8 +238,10 @@ def moe_ff(h, w, p, mlp):
 
 # ----------------------------------------------------------------------------- the model
 
-def forward(cfg, w, tokens, positions=None, taps=None):
-    """Logits [n, vocab] of one whole sequence; ``taps`` (a list) receives the stream after every layer."""
+def forward(cfg, w, tokens, positions=None, taps=None, margins=None):
+    """Logits [n, vocab] of one whole sequence; ``taps`` (a list) receives the stream after every
+    layer, ``margins`` (a list) one list a routed layer: by how much each token's closest call of
+    the router was decided."""
     n = len(tokens)
     positions = list(range(n)) if positions is None else list(positions)
     eps, m = float(cfg["norm"]["eps"]), float(cfg.get("residual_mult", 1.0))
@@ -243,8 +257,90 @@ def forward(cfg, w, tokens, positions=None, taps=None):
         mlp = layer.get("mlp")
         if mlp is not None:
             h = rms_norm(x, w[p + ".norm2"], eps)
-            y = dense_ff(h, w, p + ".mlp", mlp) if mlp["kind"] == "dense" else moe_ff(h, w, p + ".mlp", mlp)
+            if mlp["kind"] == "dense":
+                y = dense_ff(h, w, p + ".mlp", mlp)
+            else:
+                per_token = [] if margins is not None else None
+                y = moe_ff(h, w, p + ".mlp", mlp, per_token)
+                if margins is not None:
+                    margins.append(per_token)
             x = x + m * rms_norm(y, w[p + ".norm2b"], eps)
         if taps is not None:
             taps.append(x.clone())
     return rms_norm(x, w["final.norm"], eps) @ w["embed"].T
+
+
+def greedy(cfg, w, prompt, n):
+    """n tokens, each the first largest logit behind the sequence so far."""
+    seq, out = list(prompt), []
+    for _ in range(n):
+        nxt = int(torch.argmax(forward(cfg, w, seq)[-1]))
+        out.append(nxt)
+        seq.append(nxt)
+    return out
+
+
+# ----------------------------------------------------------------------------- random weights
+
+def _attention_tensors(p, m, width, g):
+    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    rn = lambda *s: torch.randn(*s, generator=g, dtype=F64)
+    return {p + ".q": rn(H * d, width) / math.sqrt(width), p + ".k": rn(G * d, width) / math.sqrt(width),
+            p + ".v": rn(G * dv, width) / math.sqrt(width), p + ".o": rn(width, H * dv) / math.sqrt(H * dv),
+            p + ".q.norm": 1.0 + 0.3 * rn(H * d), p + ".k.norm": 1.0 + 0.3 * rn(G * d)}
+
+
+def _delta_tensors(p, m, width, g, a_rank, gate_rank):
+    H, G, d, dv, taps = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
+    rn = lambda *s: torch.randn(*s, generator=g, dtype=F64)
+    return {p + ".q": rn(G * d, width) / math.sqrt(width), p + ".k": rn(G * d, width) / math.sqrt(width),
+            p + ".v": rn(H * dv, width) / math.sqrt(width), p + ".b": rn(H, width) / math.sqrt(width),
+            p + ".q.conv": rn(G * d, taps) * 0.6, p + ".k.conv": rn(G * d, taps) * 0.6, p + ".v.conv": rn(H * dv, taps) * 0.6,
+            p + ".a1": rn(a_rank, width) / math.sqrt(width), p + ".a2": rn(H * d, a_rank) / math.sqrt(a_rank) * 2.0,
+            p + ".g1": rn(gate_rank, width) / math.sqrt(width), p + ".g2": rn(H * dv, gate_rank) / math.sqrt(gate_rank) * 2.0,
+            # decays spread between forgetting at once and hardly at all
+            p + ".A_log": rn(H) * 0.8 - 0.5, p + ".dt_bias": rn(H * d) * 1.5 - 1.0,
+            p + ".norm": 1.0 + 0.3 * rn(dv), p + ".o": rn(width, H * dv) / math.sqrt(H * dv)}
+
+
+def _expert_tensors(p, ff, width, g):
+    rn = lambda *s: torch.randn(*s, generator=g, dtype=F64)
+    return {p + ".gate": rn(ff, width) / math.sqrt(width) * 1.5, p + ".up": rn(ff, width) / math.sqrt(width) * 1.5,
+            p + ".down": rn(width, ff) / math.sqrt(ff)}
+
+
+def random_weights(cfg, seed, a_rank=6, gate_rank=10):
+    """Weights of a size that keeps every mechanism in play: products of unit scale, gates that
+    reach their clamps, router scores spread over the experts."""
+    g = torch.Generator().manual_seed(seed)
+    width = cfg["width"]
+    rn = lambda *s: torch.randn(*s, generator=g, dtype=F64)
+    w = {"embed": rn(cfg["vocab"], width) / math.sqrt(width) * 2.0, "final.norm": 1.0 + 0.2 * rn(width)}
+    for i, layer in enumerate(cfg["layers"]):
+        p = f"l{i}"
+        for name in ("norm1", "norm1b"):
+            w[f"{p}.{name}"] = 1.0 + 0.2 * rn(width)
+        if layer["type"] == "parallel":
+            w.update(_attention_tensors(p + ".mix.left", layer["mixer"]["left"], width, g))
+            right = layer["mixer"]["right"]
+            w.update(_delta_tensors(p + ".mix.right", right, width, g, right.get("a_rank", a_rank),
+                                    right.get("gate_rank", gate_rank)))
+            w[p + ".mix.left.out"] = 1.0 + 0.2 * rn(width)
+            w[p + ".mix.right.out"] = 1.0 + 0.2 * rn(width)
+        else:
+            w.update(_attention_tensors(p + ".mix", layer["mixer"], width, g))
+        mlp = layer.get("mlp")
+        if mlp is None:
+            continue
+        for name in ("norm2", "norm2b"):
+            w[f"{p}.{name}"] = 1.0 + 0.2 * rn(width)
+        if mlp["kind"] == "dense":
+            w.update(_expert_tensors(p + ".mlp", mlp["ff"], width, g))
+        else:
+            for e in range(mlp["router"]["experts"]):
+                w.update(_expert_tensors(f"{p}.mlp.e{e}", mlp["expert"]["ff"], width, g))
+            w[p + ".mlp.router"] = rn(mlp["router"]["experts"], width) / math.sqrt(width) * 2.0
+            if mlp.get("shared"):
+                w.update(_expert_tensors(p + ".mlp.shared", mlp["shared"]["ff"], width, g))
+                w[p + ".mlp.shared.sg"] = rn(1, width) / math.sqrt(width) * 2.0
+    return w
