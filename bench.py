@@ -23,6 +23,8 @@ Other workloads, each printing one JSON line of its own (``--model`` chooses the
     --workload natenex         prefill and decode of a Natenex model (windowed attention that keeps the first
                                positions beside a gated linear recurrence, a gated delta rule, attention through
                                latents) beside a Nusilix and a Llama model of the same layer sizes
+    --workload lugetar         prefill and decode of a Lugetar model (attention layers in turn with layers of chunked
+                               attention beside a gated delta rule and routed experts) beside Natenex, Ribovik and Llama
     --workload nusilix         prefill and decode of a Nusilix model (every fourth layer recurrent)
                                beside a Llama model of the same layer sizes (--sizes NAME; all if
                                not given)
@@ -58,8 +60,8 @@ def main(argv=None):
     ap.add_argument("--model", default="tinyllama-1.1b", choices=["tinyllama-1.1b", "llama2-7b", "llama3-8b"],
                     help="whose sizes to run (the default is the headline configuration)")
     ap.add_argument("--extra", default="", help="engine options for experiments: key=value,key=value (ints or words)")
-    ap.add_argument("--workload", default="headline", choices=["headline", "decode-run", "prefill-chunks", "mixed", "nusilix", "ribovik", "natenex"])
-    ap.add_argument("--sizes", default="", help="layer sizes of the nusilix, ribovik and natenex workloads (see benchmark.NUSILIX_SIZES)")
+    ap.add_argument("--workload", default="headline", choices=["headline", "decode-run", "prefill-chunks", "mixed", "nusilix", "ribovik", "natenex", "lugetar"])
+    ap.add_argument("--sizes", default="", help="layer sizes of the nusilix, ribovik, natenex and lugetar workloads (see benchmark.NUSILIX_SIZES)")
     ap.add_argument("--chunk", type=int, default=512, help="tokens per prompt portion (prefill-chunks, mixed)")
     ap.add_argument("--requests", type=int, default=32, help="requests of the mixed workload")
     ap.add_argument("--new-tokens", type=int, default=64, help="tokens each request of the mixed workload generates")
@@ -94,7 +96,7 @@ def main(argv=None):
     for item in filter(None, args.extra.split(",")):
         key, _, val = item.partition("=")
         extra[key] = int(val) if val.lstrip("-").isdigit() else (val or True)
-    if args.workload in ("nusilix", "ribovik", "natenex"):
+    if args.workload in ("nusilix", "ribovik", "natenex", "lugetar"):
         names = [args.sizes] if args.sizes else sorted(B.NUSILIX_SIZES)
         res = {"workload": args.workload, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
                "weights": "random", "context": args.context}
@@ -104,7 +106,7 @@ def main(argv=None):
                 sizes["layers"] = args.layers
             res[name] = dict(sizes=sizes, **B.measure_design_pair(
                 sizes, args.dtype, context=args.context, steps=min(args.steps, 64), design=args.workload,
-                design_sizes=B.RIBOVIK_EXPERTS[name] if args.workload == "ribovik" else None))
+                design_sizes={"ribovik": B.RIBOVIK_EXPERTS, "lugetar": B.LUGETAR_EXPERTS}.get(args.workload, {}).get(name)))
         print(json.dumps(res))
         return 0
     if args.workload != "headline":

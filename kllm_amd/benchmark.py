@@ -386,6 +386,37 @@ def natenex_config(width, heads, kv_heads, head_dim, ff, layers, vocab, window=1
             "norm": {"eps": 1e-6}, "layers": [dict(cycle[i % 4]) for i in range(layers)]}
 
 
+# Lugetar beside Natenex, Ribovik and Llama: layers in turn 'attention' (Llama's heads, causal, a
+# query temperature, the dense clamped feed-forward as wide as Llama's) and 'parallel' (the same
+# heads with a rotation of half of each head behind a chunked mask of half the context, beside a
+# gated delta rule of width / 128 heads of 128 x 128 on half as many key heads whose decay and
+# output gate come through inner widths of 64 and width / 16; experts as Ribovik's, in four groups
+# of which two are kept).
+LUGETAR_EXPERTS = {
+    "1.1b-sizes": dict(experts=16, top=2, expert_ff=1408, shared_ff=1408),
+    "8b-sizes": dict(experts=8, top=2, expert_ff=3584, shared_ff=3584),
+}
+
+
+def lugetar_config(width, heads, kv_heads, head_dim, ff, layers, vocab, chunk=1024, experts=16, top=2, expert_ff=1408,
+                   shared_ff=1408) -> dict:
+    attention = {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+                 "q_temp": {"coef": 0.2, "every": 512}}
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+            "mask": {"size": chunk},
+            "rot": {"base": 500000.0, "dims": head_dim // 2,
+                    "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 1024}}}
+    right = {"heads": width // 128, "kv_heads": max(1, width // 256), "dim": 128, "vdim": 128, "conv": 4,
+             "a_rank": 64, "gate_rank": width // 16}
+    moe = {"kind": "moe", "expert": {"ff": expert_ff},
+           "router": {"experts": experts, "top": top, "scale": 2.5, "groups": {"count": 4, "keep": 2}},
+           "shared": {"ff": shared_ff}}
+    cycle = ({"type": "attention", "mixer": attention, "mlp": {"kind": "dense", "ff": ff, "limit": 7.0}},
+             {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": moe})
+    return {"architecture": "Lugetar", "vocab": vocab, "width": width, "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-6}, "residual_mult": 0.7, "layers": [dict(cycle[i % 2]) for i in range(layers)]}
+
+
 def spread_routing(eng: Engine, seed: int = 0) -> None:
     """Random weights as the engine draws them (all small, corrections all near 1) send every
     token to the same experts.  A router with large weights and no correction spreads the
@@ -406,9 +437,9 @@ def spread_routing(eng: Engine, seed: int = 0) -> None:
 
 def measure_design_pair(sizes: dict, dtype: str, batches=(1, 8), context: int = 2048, prompt: int = 2048,
                         steps: int = 64, delta_every: int = 4, design: str = "nusilix", design_sizes=None) -> dict:
-    """Prefill and decode throughput of a model of ``design`` ("nusilix", "ribovik", "natenex") and
-    of a Llama model of the same layer sizes (for Natenex a Nusilix model too, the nearest in
-    kind), one after the other on this GPU."""
+    """Prefill and decode throughput of a model of ``design`` ("nusilix", "ribovik", "natenex",
+    "lugetar") and of a Llama model of the same layer sizes (for Natenex a Nusilix model too, for
+    Lugetar a Natenex and a Ribovik model: the nearest in kind), one after the other on this GPU."""
     import gc
     out = {}
     models = []
@@ -417,6 +448,10 @@ def measure_design_pair(sizes: dict, dtype: str, batches=(1, 8), context: int = 
     elif design == "natenex":
         first = natenex_config(**sizes, window=max(64, context // 2))
         models.append(("nusilix", nusilix_config(delta_every=delta_every, **sizes)))
+    elif design == "lugetar":
+        first = lugetar_config(**sizes, **(design_sizes or {}), chunk=max(64, context // 2))
+        models.append(("natenex", natenex_config(**sizes, window=max(64, context // 2))))
+        models.append(("ribovik", ribovik_config(**sizes, chunk=max(4096, context + 64))))
     else:
         first = nusilix_config(delta_every=delta_every, **sizes)
     for name, cfg in [(design, first)] + models + [("llama", llama_config(**sizes))]:

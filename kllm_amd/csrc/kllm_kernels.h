@@ -347,7 +347,9 @@ int kllm_delta_out(const float* o, const float* gate, const float* weight, float
  * weight * N(x); N(v) = v / sqrt(mean(v^2) + eps).  `out` (or null) receives the new rows of x in
  * `out_dtype`, for the next product; with `next_weight` [d] it receives next_weight * N(x) of the
  * new rows instead: the norm in front of the next sub-layer.  `delta_scale` [n] (or null) is a
- * factor per row on delta's slices.
+ * factor per row on delta's slices.  With `pair_b` ([pair_nb][n][d]) the sums are those of two
+ * sub-layers side by side, each normed before they are added: pair_sa * pair_wa * N(delta) +
+ * pair_sb * pair_wb * N(pair_b) stands where delta's slices stood.
  * The sums may also be those of a routed feed-forward's chosen experts, not yet added up
  * (`chosen_y` [n * top][d], null: none): then the row is the sum over the token's choices of
  * chosen_wgt * (chosen_idx < E ? chosen_y : chosen_x, the feed-forward's input [n][d]) + delta's
@@ -356,7 +358,8 @@ int kllm_norm_residual(float* x, const float* delta, int nsplit, long split_stri
                        const float* weight, void* out, int out_dtype, int n, int d, float eps,
                        const float* chosen_y, const void* chosen_x, int chosen_x_dtype, const int* chosen_idx,
                        const float* chosen_wgt, int top, int E, float mult, const float* next_weight,
-                       const float* delta_scale, hipStream_t stream);
+                       const float* delta_scale, const float* pair_b, int pair_nb, long pair_stride,
+                       const float* pair_wa, const float* pair_wb, float pair_sa, float pair_sb, hipStream_t stream);
 /* cos/sin [n][half] = factor * cos/sin(positions[t] * freq[i]), the angle in double. */
 int kllm_rope_tables_freq(float* cos_t, float* sin_t, const int* positions, const double* freq, int n,
                           int half, double factor, hipStream_t stream);
@@ -442,16 +445,17 @@ int kllm_conv_state_update(const float* proj, int nsplit, long split_stride, int
  * v (H dv) | b (H) | a (H) | gate (H dv) | anything else.  conv_w [2 G dk + H dv][taps]; state: the
  * convolution's field.  Writes qn, kn [n][G dk] (unit vectors per head, qn times dk^-1/2), vv [n][H dv],
  * gb [n][2][H] (decay, beta) and gate [n][H dv] = silu of the gate's sums (`gate_sigmoid`: their
- * logistic function).  With `a_sums` ([a_ns][n][H dk], a_stride between slices) the decay has one
- * number per head and key channel, exp(-exp(a_log[h]) softplus(a + dt_bias[h][c])), written to `dec`
- * [n][H dk]; proj then has no a columns.  With `gate_sums` ([g_ns][n][H dv]) the gate's sums are
- * these and proj has no gate columns. */
+ * logistic function).  With `a_sums` ([a_ns][n][a_row], a_stride between slices, the first H dk of
+ * a row) the decay has one number per head and key channel, exp(-exp(a_log[h]) softplus(a +
+ * dt_bias[h][c])), written to `dec` [n][H dk]; proj then has no a columns.  With `gate_sums`
+ * ([g_ns][n][g_row], the first H dv of a row) the gate's sums are these and proj has no gate
+ * columns. */
 int kllm_gated_delta_prep(const float* proj, int nsplit, long split_stride, const float* conv_w, int taps,
                           const float* state, long slot_stride, const float* a_log, const float* dt_bias,
                           const int* span_of_token, const int* slots, const int* span_start, const int* span_pos,
                           float* qn, float* kn, float* vv, float* gb, float* gate, int n, int H, int G, int dk,
-                          int dv, float unit_eps, int cols, const float* a_sums, int a_ns, long a_stride,
-                          const float* gate_sums, int g_ns, long g_stride, int gate_sigmoid, float* dec,
+                          int dv, float unit_eps, int cols, const float* a_sums, int a_ns, long a_stride, int a_row,
+                          const float* gate_sums, int g_ns, long g_stride, int g_row, int gate_sigmoid, float* dec,
                           hipStream_t stream);
 int kllm_gated_delta_max_dim(void);
 /* The recurrence: state [H][dk][dv] per slot, o_out [n][H dv].  `dec` (or null): decays per head and

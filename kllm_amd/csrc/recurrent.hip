@@ -85,54 +85,79 @@ __global__ __launch_bounds__(kRecThreads) void conv_state_update_kernel(
 // ---------------------------------------------------------------------------- gated delta rule
 
 // proj: [nsplit][n][cols], columns q (G*dk) | k (G*dk) | v (H*dv) | b (H) | a (H) | gate (H*dv) |
-// whatever else the product made.  With `a_sums` ([a_ns][n][H*dk]) the decay has one number per
-// head and key channel, from sums of their own, and proj has no a columns; with `gate_sums`
-// ([g_ns][n][H*dv]) the gate's sums are their own too and proj has no gate columns.
-// One workgroup a token.  Dynamic LDS: the convolved q, k, v of the token, [2*G*dk + H*dv] floats.
+// whatever else the product made.  With `a_sums` ([a_ns][n][a_row], the first H*dk of a row) the
+// decay has one number per head and key channel, from sums of their own, and proj has no a
+// columns; with `gate_sums` ([g_ns][n][g_row], the first H*dv of a row) the gate's sums are their
+// own too and proj has no gate columns.
+// One wave per (token, item): the items are the G query heads, the G key heads and the H value
+// heads; a value head's wave also makes that head's gate, decays and beta.  A lane keeps up to
+// four channels of a query or key head (heads of up to 256) between the sum and the division.
 __global__ __launch_bounds__(kRecThreads) void gated_delta_prep_kernel(
     const float* __restrict__ proj, int nsplit, long split_stride, const float* __restrict__ conv_w, int taps,
     const float* __restrict__ state, long slot_stride, const float* __restrict__ a_log,
     const float* __restrict__ dt_bias, const int* __restrict__ span_of_token, const int* __restrict__ slots,
     const int* __restrict__ span_start, const int* __restrict__ span_pos, float* __restrict__ qn,
     float* __restrict__ kn, float* __restrict__ vv, float* __restrict__ gb, float* __restrict__ gate, int H, int G,
-    int dk, int dv, float unit_eps, long cols, const float* __restrict__ a_sums, int a_ns, long a_stride,
-    const float* __restrict__ gate_sums, int g_ns, long g_stride, int gate_sigmoid, float* __restrict__ dec) {
-  extern __shared__ float vals[];
+    int dk, int dv, float unit_eps, long cols, const float* __restrict__ a_sums, int a_ns, long a_stride, long a_row,
+    const float* __restrict__ gate_sums, int g_ns, long g_stride, long g_row, int gate_sigmoid,
+    float* __restrict__ dec) {
   const long t = blockIdx.x;
-  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int item = blockIdx.y * (kRecThreads / kWave) + threadIdx.x / kWave;
+  if (item >= 2 * G + H) return;
   const int QK = G * dk, HV = H * dv, C = 2 * QK + HV;
   const int gate_col = C + (a_sums ? H : 2 * H);
   const int span = span_of_token[t];
   const long t0 = span_start[span];
   const bool fresh = span_pos[span] == 0;
   const float* st = state + (long)slots[span] * slot_stride;
-  for (int c = tid; c < C; c += kRecThreads) {
+  auto convolved = [&](int c) {
     const float y = conv_at(proj, nsplit, split_stride, cols, c, nullptr, conv_w + (long)c * taps, taps,
                             st + (long)c * (taps - 1), fresh, t, t0);
-    vals[c] = y / (1.f + expf(-y));                       // SiLU
-  }
-  __syncthreads();
-  // a wave a head of q or k: the unit norm
-  for (int item = wave; item < 2 * G; item += kRecThreads / kWave) {
-    const float* src = vals + (long)item * dk;
+    return y / (1.f + expf(-y));                         // SiLU
+  };
+  if (item < 2 * G) {        // a head of q or k: the unit norm
+    const int c0 = item * dk;                            // q's heads, then k's, lie side by side
+    float val[4];
     float ss = 0.f;
-    for (int e = lane; e < dk; e += kWave) ss = fmaf(src[e], src[e], ss);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int e = lane + kWave * r;
+      val[r] = e < dk ? convolved(c0 + e) : 0.f;
+      ss = fmaf(val[r], val[r], ss);
+    }
     ss = wave_sum(ss);
     const bool is_q = item < G;
     const float f = (is_q ? 1.f / sqrtf((float)dk) : 1.f) / sqrtf(ss + unit_eps);
-    float* dst = (is_q ? qn + t * QK + (long)item * dk : kn + t * QK + (long)(item - G) * dk);
-    for (int e = lane; e < dk; e += kWave) dst[e] = src[e] * f;
+    float* dst = is_q ? qn + t * QK + (long)item * dk : kn + t * QK + (long)(item - G) * dk;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int e = lane + kWave * r;
+      if (e < dk) dst[e] = val[r] * f;
+    }
+    return;
   }
-  for (int c = tid; c < HV; c += kRecThreads) {
-    vv[t * HV + c] = vals[2 * QK + c];
+  const int h = item - 2 * G;
+  for (int e = lane; e < dv; e += kWave) {
+    const int c = h * dv + e;
+    vv[t * HV + c] = convolved(2 * QK + c);
     float g = 0.f;
     if (gate_sums)
-      for (int s = 0; s < g_ns; ++s) g += gate_sums[s * g_stride + t * HV + c];
+      for (int s = 0; s < g_ns; ++s) g += gate_sums[s * g_stride + t * g_row + c];
     else
       for (int s = 0; s < nsplit; ++s) g += proj[s * split_stride + t * cols + gate_col + c];
     gate[t * HV + c] = gate_sigmoid ? sigmoid_f32(g) : g / (1.f + expf(-g));
   }
-  for (int h = tid; h < H; h += kRecThreads) {
+  if (a_sums) {       // one decay per head and key channel; dt_bias has as many entries
+    const float rate = expf(a_log[h]);
+    for (int e = lane; e < dk; e += kWave) {
+      const int c = h * dk + e;
+      float a = 0.f;
+      for (int s = 0; s < a_ns; ++s) a += a_sums[s * a_stride + t * a_row + c];
+      dec[t * (long)H * dk + c] = expf(-rate * softplus_f32(a + dt_bias[c]));
+    }
+  }
+  if (lane == 0) {
     float b = 0.f, a = 0.f;
     for (int s = 0; s < nsplit; ++s) {
       b += proj[s * split_stride + t * cols + C + h];
@@ -140,14 +165,6 @@ __global__ __launch_bounds__(kRecThreads) void gated_delta_prep_kernel(
     }
     gb[t * 2 * H + h] = a_sums ? 1.f : expf(-expf(a_log[h]) * softplus_f32(a + dt_bias[h]));
     gb[t * 2 * H + H + h] = sigmoid_f32(b);
-  }
-  if (a_sums) {       // one decay per head and key channel; dt_bias has as many entries
-    const int HK = H * dk;
-    for (int c = tid; c < HK; c += kRecThreads) {
-      float a = 0.f;
-      for (int s = 0; s < a_ns; ++s) a += a_sums[s * a_stride + t * HK + c];
-      dec[t * HK + c] = expf(-expf(a_log[c / dk]) * softplus_f32(a + dt_bias[c]));
-    }
   }
 }
 
@@ -515,8 +532,9 @@ extern "C" int kllm_gated_delta_prep(const float* proj, int nsplit, long split_s
                                      const int* span_of_token, const int* slots, const int* span_start,
                                      const int* span_pos, float* qn, float* kn, float* vv, float* gb, float* gate,
                                      int n, int H, int G, int dk, int dv, float unit_eps, int cols,
-                                     const float* a_sums, int a_ns, long a_stride, const float* gate_sums, int g_ns,
-                                     long g_stride, int gate_sigmoid, float* dec, hipStream_t stream) {
+                                     const float* a_sums, int a_ns, long a_stride, int a_row, const float* gate_sums,
+                                     int g_ns, long g_stride, int g_row, int gate_sigmoid, float* dec,
+                                     hipStream_t stream) {
   KLLM_REQUIRE(proj && conv_w && state && a_log && dt_bias && span_of_token && slots && span_start && span_pos && qn &&
                    kn && vv && gb && gate, "gated_delta_prep: null pointer");
   KLLM_REQUIRE((a_sums == nullptr) == (dec == nullptr) && (!a_sums || a_ns >= 1) && (!gate_sums || g_ns >= 1),
@@ -526,12 +544,15 @@ extern "C" int kllm_gated_delta_prep(const float* proj, int nsplit, long split_s
   KLLM_REQUIRE(n > 0 && H > 0 && G > 0 && H % G == 0 && dk > 0 && dv > 0 && nsplit >= 1,
                "gated_delta_prep: bad sizes n=%d H=%d G=%d dk=%d dv=%d", n, H, G, dk, dv);
   KLLM_REQUIRE(taps >= 1 && taps <= kMaxTaps, "gated_delta_prep: %d taps (1 to %d)", taps, kMaxTaps);
-  const size_t lds = ((size_t)2 * G * dk + (size_t)H * dv) * sizeof(float);
-  KLLM_REQUIRE(lds <= 64 * 1024, "gated_delta_prep: %zu bytes of a token's channels do not fit into LDS", lds);
-  hipLaunchKernelGGL(gated_delta_prep_kernel, dim3(n), dim3(kRecThreads), lds, stream, proj, nsplit, split_stride,
-                     conv_w, taps, state, slot_stride, a_log, dt_bias, span_of_token, slots, span_start, span_pos, qn,
-                     kn, vv, gb, gate, H, G, dk, dv, unit_eps, (long)cols, a_sums, a_ns, a_stride, gate_sums, g_ns,
-                     g_stride, gate_sigmoid, dec);
+  KLLM_REQUIRE(dk <= 4 * kWave, "gated_delta_prep: key heads of %d (up to %d)", dk, 4 * kWave);
+  KLLM_REQUIRE((!a_sums || a_row >= H * dk) && (!gate_sums || g_row >= H * dv),
+               "gated_delta_prep: rows of %d and %d sums do not hold the decays and the gates", a_row, g_row);
+  const int items = 2 * G + H, per_wg = kRecThreads / kWave;
+  KLLM_REQUIRE(ceil_div(items, per_wg) <= 65535, "gated_delta_prep: %d heads are too many for the grid", items);
+  hipLaunchKernelGGL(gated_delta_prep_kernel, dim3(n, ceil_div(items, per_wg)), dim3(kRecThreads), 0, stream, proj,
+                     nsplit, split_stride, conv_w, taps, state, slot_stride, a_log, dt_bias, span_of_token, slots,
+                     span_start, span_pos, qn, kn, vv, gb, gate, H, G, dk, dv, unit_eps, (long)cols, a_sums, a_ns,
+                     a_stride, (long)a_row, gate_sums, g_ns, g_stride, (long)g_row, gate_sigmoid, dec);
   KLLM_CHECK_LAUNCH("gated_delta_prep");
   return 0;
 }

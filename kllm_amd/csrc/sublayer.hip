@@ -36,12 +36,24 @@ struct ChosenSums {
   int top, E, xin_dtype;
 };
 
+// Two sub-layers side by side whose outputs are each normed before they are added: the row is
+// sa * wa * N(delta's slices) + sb * wb * N(b's slices) in place of delta's slices.
+struct NormedPair {
+  const float* b;        // [nb][n][d], null: no such pair
+  const float* wa;       // [d]
+  const float* wb;       // [d]
+  long stride_b;
+  int nb;
+  float sa, sb;
+};
+
 template <typename TOUT, int PER>
 __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
     float* __restrict__ x, const float* __restrict__ delta, int nsplit, long split_stride,
     const float* __restrict__ bias, const float* __restrict__ w, TOUT* __restrict__ out, int d, float eps,
-    const ChosenSums chosen, float mult, const float* __restrict__ next_w, const float* __restrict__ delta_scale) {
-  extern __shared__ float row_lds[];      // [d] (PER == 0)
+    const ChosenSums chosen, float mult, const float* __restrict__ next_w, const float* __restrict__ delta_scale,
+    const NormedPair pair) {
+  extern __shared__ float row_lds[];      // [d] (PER == 0; twice that with a pair)
   __shared__ float red[16];
   const long r = blockIdx.x;
   const float dscale = delta_scale ? delta_scale[r] : 1.f;      // a factor of the row's delta (a gate of a shared expert)
@@ -103,6 +115,31 @@ __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
 #pragma unroll
           for (int j = 0; j < PER; ++j) dv[j] += src[at[j]];
         }
+        if (pair.b) {       // each of the two normed over the row before they are added
+          float bv[PER], wa[PER], wb[PER];
+#pragma unroll
+          for (int j = 0; j < PER; ++j) {
+            bv[j] = 0.f;
+            wa[j] = pair.wa[at[j]];
+            wb[j] = pair.wb[at[j]];
+          }
+          for (int s = 0; s < pair.nb; ++s) {
+            const float* src = pair.b + s * pair.stride_b + r * d;
+#pragma unroll
+            for (int j = 0; j < PER; ++j) bv[j] += src[at[j]];
+          }
+          float ssa = 0.f, ssb = 0.f;
+#pragma unroll
+          for (int j = 0; j < PER; ++j) {
+            if (threadIdx.x + kRowThreads * j >= d) dv[j] = bv[j] = 0.f;
+            ssa = fmaf(dv[j], dv[j], ssa);
+            ssb = fmaf(bv[j], bv[j], ssb);
+          }
+          const float ra = pair.sa / sqrtf(block_sum(ssa, red) / (float)d + eps);
+          const float rb = pair.sb / sqrtf(block_sum(ssb, red) / (float)d + eps);
+#pragma unroll
+          for (int j = 0; j < PER; ++j) dv[j] = fmaf(dv[j] * ra, wa[j], bv[j] * rb * wb[j]);
+        }
 #pragma unroll
         for (int j = 0; j < PER; ++j) v[j] = fmaf(dscale, dv[j], v[j]);
       }
@@ -145,12 +182,29 @@ __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
     }
     return;
   }
+  float ra = 1.f, rb = 0.f;
+  if (pair.b) {       // a pass of its own for the two sums of squares; the sums wait in LDS
+    float ssa = 0.f, ssb = 0.f;
+    for (int i = threadIdx.x; i < d; i += kRowThreads) {
+      float a = 0.f, b = 0.f;
+      for (int s = 0; s < nsplit; ++s) a += delta[s * split_stride + r * d + i];
+      for (int s = 0; s < pair.nb; ++s) b += pair.b[s * pair.stride_b + r * d + i];
+      row_lds[i] = a;
+      row_lds[d + i] = b;
+      ssa = fmaf(a, a, ssa);
+      ssb = fmaf(b, b, ssb);
+    }
+    ra = pair.sa / sqrtf(block_sum(ssa, red) / (float)d + eps);
+    rb = pair.sb / sqrtf(block_sum(ssb, red) / (float)d + eps);
+  }
   float ss = 0.f;
   for (int i = threadIdx.x; i < d; i += kRowThreads) {
     float v;
     if (sums) {
       v = chosen.y ? chosen_at(i) : 0.f;
-      if (delta) {
+      if (pair.b) {
+        v = fmaf(dscale, fmaf(row_lds[i] * ra, pair.wa[i], row_lds[d + i] * rb * pair.wb[i]), v);
+      } else if (delta) {
         float dsum = 0.f;
         for (int s = 0; s < nsplit; ++s) dsum += delta[s * split_stride + r * d + i];
         v = fmaf(dscale, dsum, v);
@@ -333,8 +387,15 @@ extern "C" int kllm_norm_residual(float* x, const float* delta, int nsplit, long
                                   const float* weight, void* out, int out_dtype, int n, int d, float eps,
                                   const float* chosen_y, const void* chosen_x, int chosen_x_dtype, const int* chosen_idx,
                                   const float* chosen_wgt, int top, int E, float mult, const float* next_weight,
-                                  const float* delta_scale, hipStream_t stream) {
+                                  const float* delta_scale, const float* pair_b, int pair_nb, long pair_stride,
+                                  const float* pair_wa, const float* pair_wb, float pair_sa, float pair_sb,
+                                  hipStream_t stream) {
   KLLM_REQUIRE(x && weight, "norm_residual: null pointer");
+  KLLM_REQUIRE(!pair_b || (delta && pair_wa && pair_wb && pair_nb >= 1 && !chosen_y),
+               "norm_residual: two normed sums come with both sums and both weights, and without chosen experts");
+  NormedPair pair;
+  pair.b = pair_b; pair.wa = pair_wa; pair.wb = pair_wb; pair.stride_b = pair_stride; pair.nb = pair_nb;
+  pair.sa = pair_sa; pair.sb = pair_sb;
   KLLM_REQUIRE(!next_weight || out, "norm_residual: the next norm's rows need a place");
   KLLM_REQUIRE(!delta_scale || delta, "norm_residual: a factor per row goes with sums");
   KLLM_REQUIRE(!chosen_y || (chosen_x && chosen_idx && chosen_wgt && top > 0 && E >= 0 &&
@@ -349,8 +410,8 @@ extern "C" int kllm_norm_residual(float* x, const float* delta, int nsplit, long
   KLLM_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "norm_residual: unknown dtype %d", out_dtype);
 #define KLLM_NR(TOUT, PER)                                                                                    \
   hipLaunchKernelGGL((norm_residual_kernel<TOUT, PER>), dim3(n), dim3(kRowThreads),                           \
-                     PER ? 0 : (size_t)d * sizeof(float), stream, x, delta, nsplit, split_stride, bias, weight, \
-                     (TOUT*)out, d, eps, chosen, mult, next_weight, delta_scale)
+                     PER ? 0 : (size_t)d * sizeof(float) * (pair_b ? 2 : 1), stream, x, delta, nsplit, split_stride, \
+                     bias, weight, (TOUT*)out, d, eps, chosen, mult, next_weight, delta_scale, pair)
   const bool bf = out && out_dtype == DT_BF16;
   if (d <= 4 * kRowThreads) {
     if (bf) KLLM_NR(bf16_t, 4); else KLLM_NR(float, 4);

@@ -21,7 +21,7 @@ import torch
 DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
 GEMV_BEST_ROWS = 0         # rows up to which they beat the MFMA kernels in bfloat16: none (a step at 1.1B sizes, one token: 1.036 against 0.963 ms)
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 
 class KernelError(RuntimeError):
@@ -113,7 +113,7 @@ def _declare(lib):
         "kllm_run_commands": [P, L, P, P],
         "kllm_fused_linear_max_parts": [],
         "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F, P, I, I, P],
-        "kllm_norm_residual": [P, P, I, L, P, P, P, I, I, I, F, P, P, I, P, P, I, I, F, P, P, P],
+        "kllm_norm_residual": [P, P, I, L, P, P, P, I, I, I, F, P, P, I, P, P, I, I, F, P, P, P, I, L, P, P, F, F, P],
         "kllm_rope_tables_freq": [P, P, P, P, I, I, D, P],
         "kllm_qkv_norm_append": [P, I, L, P, P, P, I, I, I, F, P, P, P, P, P, I, I, I, I, I, I, I, I, P, P, P],
         "kllm_gate_bias": [P, I, L, P, P, I, I, I, I, F, F, P],
@@ -149,8 +149,8 @@ def _declare(lib):
         "kllm_delta_scan": [P, P, P, P, P, P, I, I, I, I, P],
         "kllm_delta_out": [P, P, P, F, P, I, I, I, I, P],
         "kllm_conv_state_update": [P, I, L, I, I, I, P, P, L, I, P, P, P, I, P],
-        "kllm_gated_delta_prep": [P, I, L, P, I, P, L, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, P, I, L, P, I, L,
-                                  I, P, P],
+        "kllm_gated_delta_prep": [P, I, L, P, I, P, L, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, P, I, L, I, P, I, L,
+                                  I, I, P, P],
         "kllm_gated_delta_max_dim": [],
         "kllm_gated_delta_scan": [P, P, P, P, P, P, L, P, P, P, I, I, I, I, I, P, P],
         "kllm_linear_recurrence_prep": [P, I, L, P, P, P, I, P, L, P, P, P, P, P, P, P, P, P, P, P, I, I, I, P],
@@ -1383,6 +1383,15 @@ def delta_out(o, gate, weight, eps, out, heads, head_dim):
 
 # ----------------------------------------------------------------------------- norm behind the sub-layer, rotation then unit norm, routed experts
 
+class NormedPair:
+    """What two sub-layers that ran side by side leave for the norm behind them: ``scale_a *
+    weight_a * N(a) + scale_b * weight_b * N(b)``, each of the float32 sums ``a`` and ``b`` ([n, d] or
+    [slices, n, d]) normed over the row (with the eps of the norm that takes the pair)."""
+
+    def __init__(self, a, scale_a, weight_a, b, scale_b, weight_b):
+        self.a, self.scale_a, self.weight_a, self.b, self.scale_b, self.weight_b = a, float(scale_a), weight_a, b, float(scale_b), weight_b
+
+
 class ChosenSums:
     """What a routed feed-forward leaves for the norm behind it to add up: per token the weighted
     sum over its choices of ``y`` [n * top, d] (float32), or of ``xin`` [n, d] where the chosen
@@ -1401,7 +1410,7 @@ def norm_residual(x, weight, delta=None, bias=None, out=None, eps=0.0, mult=1.0,
     receives the new x in its own dtype, or, with ``next_weight`` [d], next_weight * N(new x): the
     norm in front of the next sub-layer.  ``delta_scale`` [n]: a factor per row on delta."""
     n, d = x.shape
-    chosen = None
+    chosen = pair = None
     if isinstance(delta, ChosenSums):
         chosen, delta = delta, delta.shared
         delta_scale = chosen.shared_scale if delta_scale is None else delta_scale
@@ -1409,6 +1418,11 @@ def norm_residual(x, weight, delta=None, bias=None, out=None, eps=0.0, mult=1.0,
         if (tuple(chosen.y.shape) != (n * top, d) or tuple(chosen.xin.shape) != (n, d)
                 or tuple(chosen.wgt.shape) != (n, top)):
             raise KernelError("norm_residual: the chosen experts' sums do not fit")
+    elif isinstance(delta, NormedPair):
+        pair, delta = delta, delta.a
+        pair_nb, pair_stride = _splits(pair.b, n, d, "norm_residual pair")
+        if pair.weight_a.numel() != d or pair.weight_b.numel() != d:
+            raise KernelError("norm_residual: the pair's weights do not fit")
     nsplit, stride = (1, 0) if delta is None else _splits(delta, n, d, "norm_residual")
     if weight.numel() != d or (bias is not None and bias.numel() != d) or (out is not None and tuple(out.shape) != (n, d)):
         raise KernelError("norm_residual: weight, bias or output does not fit")
@@ -1425,7 +1439,11 @@ def norm_residual(x, weight, delta=None, bias=None, out=None, eps=0.0, mult=1.0,
             _ptr(chosen.idx, "norm_residual idx", torch.int32) if chosen else 0,
             _ptr(chosen.wgt, "norm_residual wgt", F32) if chosen else 0, chosen.idx.shape[1] if chosen else 0,
             chosen.experts if chosen else 0, float(mult), _ptr(next_weight, "norm_residual next weight", F32, True),
-            _ptr(delta_scale, "norm_residual delta scale", F32, True), _stream())
+            _ptr(delta_scale, "norm_residual delta scale", F32, True),
+            _ptr(pair.b, "norm_residual pair b", F32) if pair else 0, pair_nb if pair else 0, pair_stride if pair else 0,
+            _ptr(pair.weight_a, "norm_residual pair weight", F32) if pair else 0,
+            _ptr(pair.weight_b, "norm_residual pair weight", F32) if pair else 0, pair.scale_a if pair else 0.0,
+            pair.scale_b if pair else 0.0, _stream())
 
 
 def rope_tables_freq(cos, sin, positions, freq, factor=1.0):
@@ -1627,24 +1645,37 @@ def gated_delta_max_dim() -> int:
 
 def gated_delta_prep(proj, conv_w, taps, state, conv_offset, a_log, dt_bias, span_of_token, slots, span_start, span_pos,
                      qn, kn, vv, gb, gate, heads, kv_heads, dim, vdim, unit_eps=1e-6, a_sums=None, decays=None,
-                     gate_sums=None, gate_sigmoid=False):
+                     gate_sums=None, gate_sigmoid=False, low_sums=None):
     """proj: float32 sums [nsplit, n, 2 G dk + 2 H dv + 2 H (or more)] of q | k | v | b | a | gate.
     Convolution (conv_w [2 G dk + H dv, taps], its earlier inputs from the state's field at
     ``conv_offset``) and SiLU of q, k, v; q and k to unit vectors per head, q times dk^-1/2; gb [n, 2,
     H] = (exp(-exp(a_log) softplus(a + dt_bias)), sigmoid(b)); gate [n, H dv] = silu (``gate_sigmoid``:
     the logistic function) of the gate's sums.  With ``a_sums`` (float32 sums [slices, n, H dk]) the
     decay has one number per head and key channel (dt_bias [H dk]), written to ``decays`` [n, H dk],
-    and proj has no a columns; with ``gate_sums`` ([slices, n, H dv]) proj has no gate columns."""
+    and proj has no a columns; with ``gate_sums`` ([slices, n, H dv]) proj has no gate columns.
+    ``low_sums`` ([slices, n, H dk + H dv]) is both in one: the decays' sums, then the gates'."""
     n = qn.shape[0]
     QK, HV = kv_heads * dim, heads * vdim
     C = 2 * QK + HV
     cols = proj.shape[-1]
-    need = C + (heads if a_sums is not None else 2 * heads) + (0 if gate_sums is not None else HV)
     nsplit, stride = _splits(proj, n, cols, "gated_delta_prep")
     addr, per_slot = _field(state, conv_offset, "gated_delta_prep")
     F32, I32 = torch.float32, torch.int32
-    a_ns, a_st = _splits(a_sums, n, heads * dim, "gated_delta_prep a") if a_sums is not None else (0, 0)
-    g_ns, g_st = _splits(gate_sums, n, HV, "gated_delta_prep gate") if gate_sums is not None else (0, 0)
+    a_ptr = g_ptr = a_row = g_row = 0
+    if low_sums is not None:
+        if a_sums is not None or gate_sums is not None:
+            raise KernelError("gated_delta_prep: the decays' and gates' sums come together or apart")
+        a_row = g_row = heads * dim + HV
+        a_ns, a_st = g_ns, g_st = _splits(low_sums, n, a_row, "gated_delta_prep low")
+        a_ptr = _ptr(low_sums, "gated_delta low sums", F32)
+        g_ptr = a_ptr + 4 * heads * dim
+        a_sums = gate_sums = low_sums
+    else:
+        a_ns, a_st = _splits(a_sums, n, heads * dim, "gated_delta_prep a") if a_sums is not None else (0, 0)
+        g_ns, g_st = _splits(gate_sums, n, HV, "gated_delta_prep gate") if gate_sums is not None else (0, 0)
+        a_ptr, a_row = _ptr(a_sums, "gated_delta a sums", F32, True), heads * dim
+        g_ptr, g_row = _ptr(gate_sums, "gated_delta gate sums", F32, True), HV
+    need = C + (heads if a_sums is not None else 2 * heads) + (0 if gate_sums is not None else HV)
     if (tuple(conv_w.shape) != (C, taps) or a_log.numel() != heads or cols < need
             or dt_bias.numel() != (heads * dim if a_sums is not None else heads)
             or (a_sums is None) != (decays is None) or (decays is not None and tuple(decays.shape) != (n, heads * dim))
@@ -1659,8 +1690,7 @@ def gated_delta_prep(proj, conv_w, taps, state, conv_offset, a_log, dt_bias, spa
             _ptr(span_pos, "gated_delta span_pos", I32), _ptr(qn, "gated_delta qn", F32), _ptr(kn, "gated_delta kn", F32),
             _ptr(vv, "gated_delta v", F32), _ptr(gb, "gated_delta gb", F32), _ptr(gate, "gated_delta gate", F32), n,
             int(heads), int(kv_heads), int(dim), int(vdim), float(unit_eps), int(cols),
-            _ptr(a_sums, "gated_delta a sums", F32, True), a_ns, a_st, _ptr(gate_sums, "gated_delta gate sums", F32, True),
-            g_ns, g_st, 1 if gate_sigmoid else 0, _ptr(decays, "gated_delta decays", F32, True), _stream())
+            a_ptr, a_ns, a_st, a_row, g_ptr, g_ns, g_st, g_row, 1 if gate_sigmoid else 0, _ptr(decays, "gated_delta decays", F32, True), _stream())
 
 
 def gated_delta_scan(qn, kn, vv, gb, o_out, state, offset, slots, span_start, span_pos, n_spans, heads, kv_heads, dim,

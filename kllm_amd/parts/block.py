@@ -293,8 +293,10 @@ class SandwichNormBlock(Part):
         if pending is not None:
             raise ValueError("sandwich_norm: the layer in front of it left sums pending, which it has no norm for")
         xn = call_part(self.norm_mixer, self.norm_mixer.forward, ctx, x)
-        delta = call_part(self.mixer, self.mixer.forward, ctx, xn, cache)
         behind = self.norm_mixer_out
+        # two mixers side by side whose outputs are normed before they are added: in the norm's launch
+        more = {"pair_eps": behind.eps} if getattr(self.mixer, "leaves_normed_pair", False) else {}
+        delta = call_part(self.mixer, self.mixer.forward, ctx, xn, cache, **more)
         if self.feed_forward is None:
             K.norm_residual(x, behind.weight, delta, bias=getattr(self.mixer, "out_bias", None), eps=behind.eps,
                             mult=self.mult)

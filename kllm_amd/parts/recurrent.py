@@ -74,7 +74,7 @@ class GatedDeltaMixer(Part):
             raise ValueError(f"gated_delta: gate {gate!r} is not built (silu, sigmoid)")
         self.gate_sigmoid = gate == "sigmoid"
         self.decays = self.heads * self.head_dim if self.channel_decay else self.heads    # numbers of a token's decay
-        self.w_a2 = self.w_g2 = None
+        self.w_a2 = None
         self.qk = self.kv_heads * self.head_dim
         self.hv = self.heads * self.value_dim
         self.channels = 2 * self.qk + self.hv                 # what passes the convolution
@@ -111,7 +111,8 @@ class GatedDeltaMixer(Part):
             if w("a2.weight").shape[1] != self.a_rank or w("g2.weight").shape[1] != self.gate_rank:
                 raise ValueError("gated_delta: the two halves of a low-rank projection do not fit each other")
             self.w_in = torch.cat([w(t + ".weight") for t in ("q", "k", "v", "b", "a1", "g1")], dim=0).contiguous()
-            self.w_a2, self.w_g2 = w("a2.weight"), w("g2.weight")
+            # the outer halves as one block-diagonal matrix: one product for the decays' and the gates' sums
+            self.w_a2 = torch.block_diag(w("a2.weight"), w("g2.weight")).contiguous()
         elif self.channel_decay:
             self.w_in = torch.cat([w(t + ".weight") for t in ("q", "k", "v", "b", "g")], dim=0).contiguous()
             self.w_a2 = w("a.weight")          # its sums are a product of their own
@@ -123,13 +124,12 @@ class GatedDeltaMixer(Part):
         self.norm_weight = w("norm").repeat(self.heads).contiguous()       # per channel of the concatenated heads
         self._tiled = {"in": tiled_copy(self.runtime, self.w_in, K.LINEAR_PARTS),
                        "o": tiled_copy(self.runtime, self.w_o, K.LINEAR_PARTS)}
-        for key, mat in (("a2", self.w_a2), ("g2", self.w_g2)):
-            if mat is not None:
-                self._tiled[key] = tiled_copy(self.runtime, mat, K.LINEAR_PARTS)
+        if self.w_a2 is not None:
+            self._tiled["a2"] = tiled_copy(self.runtime, self.w_a2, K.LINEAR_PARTS)
 
     def tensors(self):
-        return [t for t in (self.w_in, self.w_o, self.conv, self.a_log, self.dt_bias, self.norm_weight, self.w_a2,
-                            self.w_g2) if t is not None]
+        return [t for t in (self.w_in, self.w_o, self.conv, self.a_log, self.dt_bias, self.norm_weight, self.w_a2)
+                if t is not None]
 
     def cache_need(self):
         return CacheNeed("state", state_shape=(self.state_floats + self.channels * (self.taps - 1),))
@@ -139,8 +139,13 @@ class GatedDeltaMixer(Part):
             raise ValueError(f"gated_delta: key heads of {self.head_dim} are not built (up to {K.gated_delta_max_dim()})")
 
     def flops(self, tokens, keys_read=0.0):
-        # the projections, and per token and head three passes over the state
-        return super().flops(tokens) + 8.0 * tokens * self.heads * self.head_dim * self.value_dim
+        # the projections (of a block-diagonal matrix the blocks), and per token and head three passes over the state
+        mats = self.w_in.numel() + self.w_o.numel()
+        if self.low_rank:
+            mats += self.decays * self.a_rank + self.hv * self.gate_rank
+        elif self.w_a2 is not None:
+            mats += self.w_a2.numel()
+        return 2.0 * tokens * mats + 8.0 * tokens * self.heads * self.head_dim * self.value_dim
 
     def forward(self, ctx, xn, cache):
         n = xn.shape[0]
@@ -152,26 +157,22 @@ class GatedDeltaMixer(Part):
         gb = ctx.buf("gdelta.gb", (n, 2, self.heads), f32)
         gate = ctx.buf("gdelta.gate", (n, self.hv), f32)
         conv_at = self.state_floats
-        a_sums = gate_sums = decays = None
+        a_sums = low_sums = decays = None
         if self.low_rank:
-            # the inner halves' sums in the compute dtype, then the outer halves' products
-            first = self.channels + self.heads
-            a_in = ctx.buf("gdelta.a1", (n, self.a_rank), self.runtime.dtype)
-            g_in = ctx.buf("gdelta.g1", (n, self.gate_rank), self.runtime.dtype)
-            K.unary_act(proj, a_in, K.ACT_IDENTITY, first_column=first)
-            K.unary_act(proj, g_in, K.ACT_IDENTITY, first_column=first + self.a_rank)
-            a_sums = decode_linear(ctx, a_in, self.w_a2, "gdelta.a", self._tiled.get("a2"))
-            gate_sums = decode_linear(ctx, g_in, self.w_g2, "gdelta.g", self._tiled.get("g2"))
+            # the inner halves' sums in the compute dtype, then the outer halves' product
+            inner = ctx.buf("gdelta.inner", (n, self.a_rank + self.gate_rank), self.runtime.dtype)
+            K.unary_act(proj, inner, K.ACT_IDENTITY, first_column=self.channels + self.heads)
+            low_sums = decode_linear(ctx, inner, self.w_a2, "gdelta.low", self._tiled.get("a2"))
         elif self.channel_decay:
             a_sums = decode_linear(ctx, xn, self.w_a2, "gdelta.a", self._tiled.get("a2"))
-        if a_sums is not None and not self.channel_decay:
+        if low_sums is not None and not self.channel_decay:
             raise ValueError("gated_delta: a low-rank decay is one per head and key channel")
         if self.channel_decay:
             decays = ctx.buf("gdelta.decays", (n, self.decays), f32)
         K.gated_delta_prep(proj, self.conv, self.taps, cache.state, conv_at, self.a_log, self.dt_bias, ctx.span_of_token,
                            cache.slots, ctx.span_start, ctx.span_pos, qn, kn, vv, gb, gate, self.heads, self.kv_heads,
                            self.head_dim, self.value_dim, self.unit_eps, a_sums=a_sums, decays=decays,
-                           gate_sums=gate_sums, gate_sigmoid=self.gate_sigmoid)
+                           low_sums=low_sums, gate_sigmoid=self.gate_sigmoid)
         # (behind the launch that read the earlier inputs: the span's last ones take their place)
         K.conv_state_update(proj, 0, self.channels, self.taps, cache.state, conv_at, cache.slots, ctx.span_start,
                             ctx.span_pos, ctx.n_spans)
@@ -323,11 +324,20 @@ class MixerSum(Part):
         self.left.check_cache(page_size)
         self.right.check_cache(page_size)
 
-    def forward(self, ctx, xn, cache):
+    # With norms the two outputs can be left, not yet added, to a norm behind the mixer that has the
+    # same eps and norms each of them in its own launch (``pair_eps``: the caller's eps; it then
+    # takes a ``kernels.NormedPair``).
+    @property
+    def leaves_normed_pair(self):
+        return self.norm_eps is not None
+
+    def forward(self, ctx, xn, cache, pair_eps=None):
         views = list(cache) if isinstance(cache, (list, tuple)) else [cache]
         take = lambda m: views.pop(0) if m.cache_need() is not None else None
         left = call_part(self.left, self.left.forward, ctx, xn, take(self.left))
         right = call_part(self.right, self.right.forward, ctx, xn, take(self.right))
+        if self.norm_eps is not None and pair_eps == self.norm_eps:
+            return K.NormedPair(left, self.left_scale, self.left_norm, right, self.right_scale, self.right_norm)
         out = ctx.buf("mixer_sum.out", (xn.shape[0], left.shape[-1]), torch.float32)
         if self.norm_eps is not None:
             K.normed_sum(out, left, self.left_scale, self.left_norm, right, self.right_scale, self.right_norm, self.norm_eps)

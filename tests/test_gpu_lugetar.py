@@ -290,13 +290,21 @@ def test_delta_rule_with_a_decay_per_key_channel(H, G, dk, dv):
 def test_sum_of_two_normed_mixers():
     from kllm_amd import kernels as K
     g = torch.Generator().manual_seed(3)
-    for n, d in ((5, 37), (2, 3000)):
+    for n, d in ((5, 37), (2, 3000), (3, 4500)):
         a, b = torch.randn(2, n, d, generator=g), torch.randn(n, d, generator=g) * 3.0
         wa, wb = torch.randn(d, generator=g), torch.randn(d, generator=g)
         out = torch.empty(n, d, device="cuda")
         K.normed_sum(out, a.cuda(), 0.5, wa.cuda(), b.cuda(), 0.25, wb.cuda(), 1e-4)
         want = 0.5 * P.rms_norm(a.double().sum(0), wa.double(), 1e-4) + 0.25 * P.rms_norm(b.double(), wb.double(), 1e-4)
         assert rel(out.cpu(), want) < 2e-6
+        # the same left to the norm behind the mixer, which also makes the next norm's rows
+        x = torch.randn(n, d, generator=g)
+        w1, w2 = 1.0 + 0.3 * torch.randn(d, generator=g), 1.0 + 0.3 * torch.randn(d, generator=g)
+        new = x.double() + 0.7 * P.rms_norm(want, w1.double(), 1e-4)
+        xd, nxt = x.clone().cuda(), torch.empty(n, d, device="cuda")
+        K.norm_residual(xd, w1.cuda(), K.NormedPair(a.cuda(), 0.5, wa.cuda(), b.cuda(), 0.25, wb.cuda()), eps=1e-4, mult=0.7,
+                        out=nxt, next_weight=w2.cuda())
+        assert rel(xd.cpu(), new) < 2e-6 and rel(nxt.cpu(), P.rms_norm(new, w2.double(), 1e-4)) < 2e-6
 
 
 @pytest.mark.parametrize("E,top,groups,keep", [(8, 3, 4, 2), (6, 2, 3, 1), (16, 4, 4, 3), (6, 2, 6, 3), (5, 1, 1, 1),
