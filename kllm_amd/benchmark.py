@@ -404,17 +404,17 @@ def lugetar_config(width, heads, kv_heads, head_dim, ff, layers, vocab, chunk=10
                  "q_temp": {"coef": 0.2, "every": 512}}
     left = {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
             "mask": {"size": chunk},
-            "rot": {"base": 500000.0, "dims": head_dim // 2,
-                    "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 1024}}}
+            "rot": {"base": 1000000.0, "dims": head_dim // 2,
+                    "scaling": {"factor": 4.0, "low": 1.0, "high": 8.0, "original": 2048}}}
     right = {"heads": width // 128, "kv_heads": max(1, width // 256), "dim": 128, "vdim": 128, "conv": 4,
              "a_rank": 64, "gate_rank": width // 16}
     moe = {"kind": "moe", "expert": {"ff": expert_ff},
-           "router": {"experts": experts, "top": top, "scale": 2.5, "groups": {"count": 4, "keep": 2}},
+           "router": {"experts": experts, "top": top, "scale": 2.0, "groups": {"count": 4, "keep": 2}},
            "shared": {"ff": shared_ff}}
     cycle = ({"type": "attention", "mixer": attention, "mlp": {"kind": "dense", "ff": ff, "limit": 7.0}},
              {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": moe})
     return {"architecture": "Lugetar", "vocab": vocab, "width": width, "embedding": {"scale": 1.0},
-            "norm": {"eps": 1e-6}, "residual_mult": 0.7, "layers": [dict(cycle[i % 2]) for i in range(layers)]}
+            "norm": {"eps": 1e-5}, "residual_mult": 0.5, "layers": [dict(cycle[i % 2]) for i in range(layers)]}
 
 
 def spread_routing(eng: Engine, seed: int = 0) -> None:

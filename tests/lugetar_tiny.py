@@ -101,14 +101,14 @@ CONFIGS = {
     "G5": _cfg(77, 64, 1e-3, 1.0, 0.9, [
         layer("attention", attn(2, 2, 32, rot=32, base=100.0, chunk=16, temp=(0.2, 7)), moe(6, 2, 16, groups=(6, 3))),
         parallel(attn(2, 1, 32), delta(1, 1, 128, 128, 4), dense(40, 5.0))]),
-    "A1": _cfg(50, 32, 1e-5, 2.0, 0.7, [layer("attention", attn(4, 2, 24, vdim=40, temp=(0.3, 16)))]),
-    "P1": _cfg(50, 40, 1e-5, 2.0, 0.7, [parallel(attn(2, 1, 48, vdim=16, rot=24, chunk=20), delta(4, 2, 24, 40, 4))]),
+    "A1": _cfg(50, 32, 1e-5, 2.0, 0.65, [layer("attention", attn(4, 2, 24, vdim=40, temp=(0.3, 16)))]),
+    "P1": _cfg(50, 40, 1e-5, 2.0, 0.75, [parallel(attn(2, 1, 48, vdim=16, rot=24, chunk=20), delta(4, 2, 24, 40, 4))]),
 }
 
 # Sizes nearer to a real model's layers: heads of 64 and 128 on the matrix cores' kernels, delta
 # heads of 64 x 96 and 128 x 128, sixteen experts.
-CONFIGS["G6"] = _cfg(200, 192, 1e-6, 1.5, 0.7, [
-    layer("attention", attn(6, 2, 64, temp=(0.3, 100)), dense(160, 1.5)),
+CONFIGS["G6"] = _cfg(200, 192, 1e-6, 1.5, 0.6, [
+    layer("attention", attn(6, 2, 64, temp=(0.35, 100)), dense(160, 1.75)),
     parallel(attn(6, 2, 64, rot=32, base=30000.0, scaling=(6.0, 1.0, 4.0, 64), chunk=48), delta(6, 3, 64, 96, 4),
              moe(16, 4, 48, groups=(4, 3), scale=2.0, shared=64)),
     parallel(attn(4, 4, 128, rot=128, base=30000.0, chunk=80), delta(2, 1, 128, 128, 4), dense(128, 1.0))])

@@ -64,9 +64,9 @@ def test_choice_of_experts_within_groups():
 
 def test_clamped_gate():
     g, u = torch.tensor([-3.0, 0.5, 4.0], dtype=F64), torch.tensor([5.0, -5.0, 0.25], dtype=F64)
-    got = P.clamped_gate(g, u, 1.5)
-    want = [-3.0 / (1 + math.exp(1.702 * 3.0)) * 2.5, 0.5 / (1 + math.exp(-1.702 * 0.5)) * -0.5,
-            1.5 / (1 + math.exp(-1.702 * 1.5)) * 1.25]
+    got = P.clamped_gate(g, u, 2.0)
+    want = [-3.0 / (1 + math.exp(1.702 * 3.0)) * 3.0, 0.5 / (1 + math.exp(-1.702 * 0.5)) * -1.0,
+            2.0 / (1 + math.exp(-1.702 * 2.0)) * 1.25]
     assert torch.allclose(got, torch.tensor(want, dtype=F64))
 
 
