@@ -133,6 +133,61 @@ for _name in ("G1", "G2", "G3", "G4", "G5", "G6"):
     CONFIGS[_name + "n"] = without_choice(CONFIGS[_name])
 
 
+def random_config(seed):
+    """A configuration drawn from a seed: two to five layers in any order, every size and constant
+    drawn anew (also the values that configurations written by hand tend to make equal or 1)."""
+    import random
+    r = random.Random(seed)
+    pick = r.choice
+
+    def attention(left):
+        kv = pick([1, 2, 3, 4])
+        heads = kv * pick([1, 2, 3])
+        dim = pick([8, 12, 16, 24, 32, 40, 64, 128])
+        a = attn(heads, kv, dim, vdim=pick([dim, dim, 8, 20, 48]), scale=r.uniform(0.6, 1.6) * dim ** -0.5)
+        if r.random() < (0.8 if left else 0.3):
+            dims = pick([d for d in (4, 8, dim // 2, dim) if d <= dim and d % 2 == 0])
+            a["rot"] = {"base": pick([50.0, 1000.0, 500000.0]), "dims": dims}
+            if r.random() < 0.6:
+                low = pick([1.0, 2.0])
+                a["rot"]["scaling"] = {"factor": pick([2.0, 8.0, 32.0]), "low": low, "high": low + pick([1.0, 3.0]),
+                                       "original": pick([16, 64, 256])}
+        if r.random() < (0.85 if left else 0.3):
+            a["mask"] = {"size": pick([1, 5, 16, 23, 32, 50, 64, 100])}
+        if r.random() < (0.3 if left else 0.85):
+            a["q_temp"] = {"coef": r.uniform(0.05, 0.6), "every": pick([1, 3, 16, 64, 1000])}
+        return a
+
+    def feed_forward():
+        kind = pick(["dense", "dense", "moe", "moe", None])
+        if kind is None:
+            return None
+        if kind == "dense":
+            return dense(pick([16, 40, 72, 130]), pick([0.5, 1.0, 3.0, 20.0]))
+        count = pick([1, 2, 3, 4])
+        experts = count * pick([1, 2, 3, 4])
+        keep = r.randint(1, count)
+        top = r.randint(1, experts // count * keep)
+        return moe(experts, top, pick([8, 24, 50]), groups=(count, keep) if r.random() < 0.8 else None,
+                   scale=pick([None, 1.0, 0.5, 3.0]), shared=pick([None, 16, 36]))
+
+    layers = []
+    for _ in range(r.randint(2, 5)):
+        if r.random() < 0.5:
+            layers.append(layer("attention", attention(False), feed_forward()))
+        else:
+            kv = pick([1, 2, 4])
+            right = delta(kv * pick([1, 2, 3]), kv, pick([8, 16, 20, 32, 64]), pick([8, 16, 24, 64]), pick([1, 2, 3, 4, 6]))
+            layers.append(parallel(attention(True), right, feed_forward()))
+    cfg = _cfg(pick([40, 97, 256]), pick([24, 32, 50, 64, 96]), pick([1e-6, 1e-5, 1e-3]), pick([1.0, 3.0, 11.0]),
+               pick([1.0, 0.4, 1.4]), layers)
+    for entry in cfg["layers"]:          # a router without groups may choose among all its experts
+        mlp = entry["mlp"]
+        if mlp and mlp["kind"] == "moe" and "groups" not in mlp["router"]:
+            mlp["router"]["top"] = r.randint(1, mlp["router"]["experts"])
+    return cfg
+
+
 def write_model(out_dir, cfg, seed, store="float32", weights=None):
     """A model folder written with the safetensors library."""
     from safetensors.torch import save_file

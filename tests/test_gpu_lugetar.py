@@ -518,6 +518,25 @@ def test_whole_prompts_decoding_portions_and_mixed_batches(folders, name, length
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_configurations_drawn_from_a_seed(folders, seed, dtype):
+    """Layer orders, sizes and constants that nobody chose (in float32 every position is bound; in
+    bfloat16 the routers choose every expert): whole prompts and a mixed trace with portions down to
+    two tokens beside single tokens."""
+    name = f"R{seed}{dtype[0]}"
+    T.CONFIGS[name] = T.random_config(seed) if dtype == "float32" else T.without_choice(T.random_config(seed))
+    cfg, d = T.CONFIGS[name], folders(name, seed=seed + 100)
+    reqs = make_requests(cfg, [70, 3, 141, 18, 33], seed)
+    want = expected(d, cfg, reqs, dtype)
+    steps = traces.whole(reqs)
+    rows, _ = replay(d, dtype, steps, traces.peak_tokens(steps))
+    compare(rows, want, dtype, reqs)
+    steps, peak = traces.mixed(reqs, seed=seed, max_live=4, tail=9, max_portion=17)
+    rows, _ = replay(d, dtype, steps, peak)
+    compare(rows, want, dtype, reqs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["G1", "G6"])
 def test_a_batch_against_each_request_alone(folders, name, dtype):
     """The logits of a request do not depend on what else the step holds, beyond rounding: a
